@@ -1,0 +1,252 @@
+"""The cache manager: pages and block tables for every request and cache group, and a slot
+for each request's fixed-size state.  Host side only (no torch).
+
+Layers whose caches have the same needs form a group with pages of its own: all layers that
+keep every key are one group, layers with a window of w keys another.  A request has one
+block table per group: entry i is the page that holds positions [i*page, (i+1)*page), or -1
+where the window has passed and the page was given back.  Pages are given back when a
+request is released and when a window has passed them, and are taken again from the head of
+the free list.
+
+Reference: nanovllm/engine/block_manager.py:26-120 (one group, all keys, prefix hashes).
+The prefix-hash reuse of the reference is kept for models whose only cache is one group of
+all keys; where a window or per-request state exists, a hashed page would not carry all a
+request needs, and hits are switched off.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import numpy as np
+import xxhash
+
+from .pages import OutOfPages, PageError, PagePool, SlotPool
+
+
+@dataclass(frozen=True)
+class CacheGroup:
+    window: Optional[int]          # None: all keys
+    runs: Tuple[int, ...]          # entries of the model's order that keep their cache here
+
+
+@dataclass
+class RequestCache:
+    tables: List[List[int]]        # per group
+    num_tokens: int = 0            # positions reserved so far
+    state_slot: int = -1
+    # chain of prefix hashes of the full pages registered so far (group 0 only)
+    hashes: List[int] = field(default_factory=list)
+
+
+def plan_groups(needs) -> Tuple[List[CacheGroup], List[int]]:
+    """From the per-run needs (PagedKV / FixedState / None) the page groups, and the runs
+    that keep fixed state.  A need is recognised by its attributes, so that this module
+    imports nothing from the parts."""
+    by_window: Dict[Optional[int], List[int]] = {}
+    state_runs: List[int] = []
+    for i, need in enumerate(needs):
+        if need is None:
+            continue
+        if hasattr(need, "tensors"):
+            state_runs.append(i)
+        elif hasattr(need, "num_kv_heads"):
+            by_window.setdefault(need.window, []).append(i)
+        else:
+            raise ValueError(f"run {i}: unknown cache need {need!r}")
+    keys = sorted(by_window, key=lambda w: (w is not None, w or 0))       # the all-keys group first
+    return [CacheGroup(w, tuple(by_window[w])) for w in keys], state_runs
+
+
+def chain_hash(tokens: Sequence[int], prefix: int = -1) -> int:
+    """block_manager.py:35-41: xxh64 over the previous block's hash (8 bytes, little endian)
+    and the block's token ids as 64-bit integers."""
+    h = xxhash.xxh64()
+    if prefix != -1:
+        h.update(prefix.to_bytes(8, "little"))
+    h.update(np.asarray(tokens, dtype=np.int64).tobytes())
+    return h.intdigest()
+
+
+class CacheManager:
+    def __init__(self, groups: Sequence[CacheGroup], page_size: int, num_pages, num_state_slots: int = 0,
+                 has_state: bool = False, enable_prefix_caching: bool = True):
+        self.groups = list(groups)
+        self.page_size = page_size
+        counts = list(num_pages) if isinstance(num_pages, (list, tuple)) else [num_pages] * len(self.groups)
+        if len(counts) != len(self.groups):
+            raise ValueError("one page count per group is needed")
+        self.pools = [PagePool(n, page_size) for n in counts]
+        self.slots = SlotPool(num_state_slots)
+        self.has_state = has_state
+        self.prefix_caching = (enable_prefix_caching and not has_state and len(self.groups) == 1
+                               and self.groups[0].window is None)
+        self.requests: Dict[Hashable, RequestCache] = {}
+
+    # ------------------------------------------------------------------ requests
+    def admit(self, request: Hashable) -> RequestCache:
+        if request in self.requests:
+            raise PageError(f"request {request!r} is admitted already")
+        slot = self.slots.take() if self.slots.num_slots else -1
+        rc = RequestCache(tables=[[] for _ in self.groups], state_slot=slot)
+        self.requests[request] = rc
+        return rc
+
+    def release(self, request: Hashable) -> None:
+        """Gives back everything the request holds.  Tables are walked from the end so that a
+        request's last pages are reused before its first (block_manager.py:94-101)."""
+        rc = self.requests.pop(request)
+        for pool, table in zip(self.pools, rc.tables):
+            for page in reversed(table):
+                if page >= 0:
+                    pool.give_back(page)
+        if rc.state_slot >= 0:
+            self.slots.give_back(rc.state_slot)
+
+    def table(self, request: Hashable, group: int) -> List[int]:
+        return self.requests[request].tables[group]
+
+    # ------------------------------------------------------------------ pages for new tokens
+    def _first_needed_page(self, group: int, first_query: int) -> int:
+        w = self.groups[group].window
+        if w is None:
+            return 0
+        return max(0, first_query - w + 1) // self.page_size
+
+    def pages_needed(self, request: Hashable, new_len: int, first_query: Optional[int] = None) -> List[int]:
+        """Per group: the pages that must be taken so that positions < new_len are covered,
+        for a step whose first query stands at position first_query (default: the first
+        position not yet reserved)."""
+        rc = self.requests[request]
+        first_query = rc.num_tokens if first_query is None else first_query
+        want = (new_len + self.page_size - 1) // self.page_size
+        out = []
+        for g, table in enumerate(rc.tables):
+            lo = max(len(table), self._first_needed_page(g, first_query))
+            out.append(max(0, want - lo))
+        return out
+
+    def can_reserve(self, request: Hashable, new_len: int, first_query: Optional[int] = None) -> bool:
+        need = self.pages_needed(request, new_len, first_query)
+        give = self._passed_pages(request, first_query)
+        return all(pool.num_free + g >= n for pool, n, g in zip(self.pools, need, give))
+
+    def _passed_pages(self, request, first_query) -> List[int]:
+        rc = self.requests[request]
+        first_query = rc.num_tokens if first_query is None else first_query
+        out = []
+        for g, table in enumerate(rc.tables):
+            upto = min(self._first_needed_page(g, first_query), len(table))
+            out.append(sum(1 for p in table[:upto] if p >= 0 and self.pools[g].ref_count[p] == 1))
+        return out
+
+    def reserve(self, request: Hashable, new_len: int, first_query: Optional[int] = None) -> None:
+        """Makes the block tables cover positions < new_len.  Pages that the window has
+        passed (every position before first_query - window + 1) are given back first.
+        Raises OutOfPages, leaving the request as it was, if a pool cannot give enough."""
+        rc = self.requests[request]
+        first_query = rc.num_tokens if first_query is None else first_query
+        if not self.can_reserve(request, new_len, first_query):
+            raise OutOfPages(f"request {request!r}: not enough free pages for {new_len} tokens")
+        want = (new_len + self.page_size - 1) // self.page_size
+        for g, (pool, table) in enumerate(zip(self.pools, rc.tables)):
+            first_page = self._first_needed_page(g, first_query)
+            for i in range(min(first_page, len(table))):
+                if table[i] >= 0:
+                    pool.give_back(table[i])
+                    table[i] = -1
+            while len(table) < want:
+                table.append(pool.take() if len(table) >= first_page else -1)
+        rc.num_tokens = max(rc.num_tokens, new_len)
+
+    # ------------------------------------------------------------------ prefix reuse
+    def match_prefix(self, tokens: Sequence[int]) -> Tuple[int, List[int]]:
+        """How many leading full pages of `tokens` are in the cache already, and which pages:
+        the chain of hashes is followed until the first miss.  The last page of a request is
+        never taken from the cache, so that at least one token is computed
+        (block_manager.py:62-68)."""
+        if not self.prefix_caching:
+            return 0, []
+        pool, ps = self.pools[0], self.page_size
+        num_pages = (len(tokens) + ps - 1) // ps
+        h, pages = -1, []
+        for i in range(num_pages - 1):
+            block = tokens[i * ps:(i + 1) * ps]
+            h = chain_hash(block, h)
+            page = pool.lookup(h, block)
+            if page == -1:
+                break
+            pages.append(page)
+        return len(pages), pages
+
+    def can_admit(self, tokens: Sequence[int]) -> int:
+        """-1 if the pages for all of `tokens` are not free, else the number of leading pages
+        found in the cache (block_manager.py:58-73): a hit on a page in use costs no free
+        page, a hit on a free page still takes it off the free list."""
+        hits, pages = self.match_prefix(tokens)
+        want = (len(tokens) + self.page_size - 1) // self.page_size
+        for g, pool in enumerate(self.pools):
+            need = want
+            if g == 0:
+                need -= sum(1 for p in pages if not pool.is_free(p))
+            if pool.num_free < need:
+                return -1
+        if self.slots.num_slots and not self.slots.num_free:
+            return -1
+        return hits
+
+    def admit_with_prefix(self, request: Hashable, tokens: Sequence[int]) -> int:
+        """Admits a request, shares the cached leading pages of `tokens` and reserves the
+        rest (block_manager.py:75-92).  Returns the number of tokens already in the cache."""
+        hits, pages = self.match_prefix(tokens)
+        rc = self.admit(request)
+        try:
+            pool = self.pools[0]
+            h = -1
+            for i, page in enumerate(pages):
+                pool.share(page)
+                rc.tables[0].append(page)
+                h = chain_hash(tokens[i * self.page_size:(i + 1) * self.page_size], h)
+                rc.hashes.append(h)
+            cached = hits * self.page_size
+            rc.num_tokens = cached
+            self.reserve(request, len(tokens), first_query=cached)
+        except Exception:
+            self.release(request)
+            raise
+        return cached
+
+    def register_full_pages(self, request: Hashable, tokens: Sequence[int], computed: int) -> None:
+        """After a step: pages of the request that are now wholly computed get their chained
+        hash, so that later requests find them (block_manager.py:110-120).  `computed` is the
+        number of the request's leading tokens whose keys are in the cache."""
+        if not self.prefix_caching:
+            return
+        rc = self.requests[request]
+        pool, ps = self.pools[0], self.page_size
+        for i in range(len(rc.hashes), computed // ps):
+            block = tokens[i * ps:(i + 1) * ps]
+            h = chain_hash(block, rc.hashes[-1] if rc.hashes else -1)
+            rc.hashes.append(h)
+            pool.register(rc.tables[0][i], h, block)
+
+    # ------------------------------------------------------------------ checks
+    def check(self) -> None:
+        """Raises PageError unless every page is either free or held by exactly as many
+        block tables as its reference count says, and every slot likewise."""
+        for g, pool in enumerate(self.pools):
+            holders: Dict[int, int] = {}
+            for rc in self.requests.values():
+                seen = set()
+                for page in rc.tables[g]:
+                    if page >= 0:
+                        if page in seen:
+                            raise PageError(f"page {page} appears twice in one block table")
+                        seen.add(page)
+                        holders[page] = holders.get(page, 0) + 1
+            pool.check(holders)
+        held = sorted(rc.state_slot for rc in self.requests.values() if rc.state_slot >= 0)
+        if len(held) != len(set(held)):
+            raise PageError("a state slot is held by two requests")
+        if self.slots.num_slots and len(held) + self.slots.num_free != self.slots.num_slots:
+            raise PageError("state slots were lost")

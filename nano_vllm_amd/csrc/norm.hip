@@ -1,0 +1,115 @@
+// RMS normalisation over the last dimension, alone and fused with the residual sum.
+//
+//   rms_norm:      y = cast(x * rsqrt(mean(x^2) + eps)) * w
+//   add_rms_norm:  s = x + r;  r <- cast(s);  y = cast(s * rsqrt(mean(s^2) + eps)) * w
+//
+// as nanovllm/layers/layernorm.py:16-40 computes them: square, mean, rsqrt and scaling in
+// float, the cast to the element type before the product with the weight, and the variance
+// of the unrounded sum.  One block per row.  The weight is stored as elements or as float.
+#include "common.h"
+
+template <typename T, bool ADD, bool VEC>
+__global__ void __launch_bounds__(256)
+rms_norm_kernel(const T* x, int64_t x_stride, T* residual, int64_t r_stride,
+                const void* __restrict__ weight, int w_is_f32, T* y, int64_t y_stride,
+                int width, float eps) {
+    __shared__ float scratch[16];
+    const int64_t row = blockIdx.x;
+    const T* xr = x + row * x_stride;
+    T* rr = ADD ? residual + row * r_stride : nullptr;
+    T* yr = y + row * y_stride;
+    const T* w_e = static_cast<const T*>(weight);
+    const float* w_f = static_cast<const float*>(weight);
+
+    float ss = 0.f;
+    if (VEC) {
+        for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+            float a[8];
+            load8(xr + i, a);
+            if (ADD) {
+                float b[8];
+                load8(rr + i, b);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) a[j] += b[j];
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ss += a[j] * a[j];
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) {
+            float a = to_float(xr[i]);
+            if (ADD) a += to_float(rr[i]);
+            ss += a * a;
+        }
+    }
+    ss = block_sum(ss, scratch);
+    const float scale = rsqrtf(ss / (float)width + eps);
+
+    if (VEC) {
+        for (int i = threadIdx.x * 8; i < width; i += blockDim.x * 8) {
+            float a[8], w[8];
+            load8(xr + i, a);
+            if (ADD) {
+                float b[8];
+                load8(rr + i, b);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) a[j] += b[j];
+                store8(rr + i, a);
+            }
+            if (w_is_f32) load8(w_f + i, w); else load8(w_e + i, w);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) a[j] = round_through<T>(a[j] * scale) * w[j];
+            store8(yr + i, a);
+        }
+    } else {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) {
+            float a = to_float(xr[i]);
+            if (ADD) {
+                a += to_float(rr[i]);
+                rr[i] = from_float<T>(a);
+            }
+            const float w = w_is_f32 ? w_f[i] : to_float(w_e[i]);
+            yr[i] = from_float<T>(round_through<T>(a * scale) * w);
+        }
+    }
+}
+
+template <bool ADD>
+static int launch(const elem_t* x, int64_t x_stride, elem_t* residual, int64_t r_stride,
+                  const void* weight, int w_is_f32, elem_t* y, int64_t y_stride,
+                  int64_t rows, int width, float eps, hipStream_t stream) {
+    if (rows == 0) return 0;
+    if (rows < 0 || width <= 0) return nva_fail("rms_norm: bad shape rows=%lld width=%d", (long long)rows, width);
+    if (rows > 0x7fffffff) return nva_fail("rms_norm: too many rows (%lld)", (long long)rows);
+    const size_t vec_bytes = 8 * sizeof(elem_t);
+    const bool vec = width % 8 == 0 && x_stride % 8 == 0 && y_stride % 8 == 0 && r_stride % 8 == 0 &&
+                     nva_aligned(x, vec_bytes) && nva_aligned(y, vec_bytes) &&
+                     (!ADD || nva_aligned(residual, vec_bytes)) &&
+                     nva_aligned(weight, w_is_f32 ? 32 : vec_bytes);
+    const int threads = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
+    if (vec)
+        hipLaunchKernelGGL((rms_norm_kernel<elem_t, ADD, true>), dim3((unsigned)rows), dim3(threads), 0, stream,
+                           x, x_stride, residual, r_stride, weight, w_is_f32, y, y_stride, width, eps);
+    else
+        hipLaunchKernelGGL((rms_norm_kernel<elem_t, ADD, false>), dim3((unsigned)rows), dim3(threads), 0, stream,
+                           x, x_stride, residual, r_stride, weight, w_is_f32, y, y_stride, width, eps);
+    return nva_check_launch("rms_norm");
+}
+
+// y may be x.  Strides are in elements between rows.
+NVA_EXPORT int NVA_NAME(nva_rms_norm)(const void* x, int64_t x_stride, const void* weight, int w_is_f32,
+                                      void* y, int64_t y_stride, int64_t rows, int width, float eps,
+                                      hipStream_t stream) {
+    return launch<false>((const elem_t*)x, x_stride, nullptr, 0, weight, w_is_f32, (elem_t*)y, y_stride,
+                         rows, width, eps, stream);
+}
+
+// residual is updated in place with the sum; y may be x.
+NVA_EXPORT int NVA_NAME(nva_add_rms_norm)(const void* x, int64_t x_stride, void* residual, int64_t r_stride,
+                                          const void* weight, int w_is_f32, void* y, int64_t y_stride,
+                                          int64_t rows, int width, float eps, hipStream_t stream) {
+    return launch<true>((const elem_t*)x, x_stride, (elem_t*)residual, r_stride, weight, w_is_f32,
+                        (elem_t*)y, y_stride, rows, width, eps, stream);
+}
+
+NVA_DEFINE_LAST_ERROR(nva_norm)

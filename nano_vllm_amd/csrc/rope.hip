@@ -1,0 +1,155 @@
+// Position encoding and the write into the paged cache, in one pass over a step's q, k and v.
+//
+// For every token and head of the packed projection row [q heads | k heads | v heads]:
+//   q, k:  optional per-head RMS norm over the head (nanovllm/models/qwen3.py:68-70,82-84),
+//          then the rotation of pairs (i, i + rot/2) by the angle table's row of the token's
+//          position (nanovllm/layers/rotary_embedding.py:6-14,44-47), in float, one rounding;
+//          q is written back in place, k in place and into its page slot;
+//   v:     copied into its page slot (nanovllm/layers/attention.py:10-30), stored transposed.
+// Cache layouts:  K [pages, kv_heads, page_size, head_dim],  V [pages, kv_heads, head_dim, page_size].
+// slot = page * page_size + offset; slot -1 writes nothing into the cache.
+#include "common.h"
+
+// table[p, 0:half] = cos(p * inv_freq), table[p, half:2*half] = sin(p * inv_freq); the product
+// p * inv_freq is one float multiplication, as the reference's outer product
+// (rotary_embedding.py:30-31).
+__global__ void rotary_table_kernel(const float* __restrict__ inv_freq, int half, int64_t positions,
+                                    float* __restrict__ table) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= positions * half) return;
+    const int64_t p = idx / half;
+    const int i = (int)(idx % half);
+    const float angle = (float)p * inv_freq[i];
+    table[p * 2 * half + i] = cosf(angle);
+    table[p * 2 * half + half + i] = sinf(angle);
+}
+
+NVA_EXPORT int NVA_NAME(nva_rotary_table)(const float* inv_freq, int half, int64_t positions, float* table,
+                                          hipStream_t stream) {
+    if (half <= 0 || positions <= 0) return nva_fail("rotary_table: bad shape half=%d positions=%lld", half, (long long)positions);
+    const int64_t n = positions * half;
+    hipLaunchKernelGGL(rotary_table_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, inv_freq, half,
+                       positions, table);
+    return nva_check_launch("rotary_table");
+}
+
+#define NVA_MAX_PER_LANE 4   // head_dim / 2 <= 64 * 4
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, int num_q_heads, int num_kv_heads, int head_dim,
+                          const void* __restrict__ q_weight, const void* __restrict__ k_weight, int w_is_f32,
+                          float eps, const float* __restrict__ table,
+                          const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
+                          T* k_cache, T* v_cache, int page_size) {
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x % NVA_WAVE;
+    const int head = blockIdx.y * (blockDim.x / NVA_WAVE) + threadIdx.x / NVA_WAVE;
+    const int total_heads = num_q_heads + 2 * num_kv_heads;
+    if (head >= total_heads) return;
+    T* row = qkv + t * row_stride + (int64_t)head * head_dim;
+    const int64_t slot = slots ? slots[t] : -1;
+    const int half = head_dim / 2;
+
+    if (head >= num_q_heads + num_kv_heads) {                       // a v head: copy, transposed
+        if (slot < 0 || !v_cache) return;
+        const int h = head - num_q_heads - num_kv_heads;
+        const int64_t page = slot / page_size, off = slot % page_size;
+        T* dst = v_cache + ((page * num_kv_heads + h) * (int64_t)head_dim) * page_size + off;
+        for (int d = lane; d < head_dim; d += NVA_WAVE) dst[(int64_t)d * page_size] = row[d];
+        return;
+    }
+
+    const bool is_q = head < num_q_heads;
+    const void* weight = is_q ? q_weight : k_weight;
+    float x1[NVA_MAX_PER_LANE], x2[NVA_MAX_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < NVA_MAX_PER_LANE; ++j) {
+        const int i = lane + j * NVA_WAVE;
+        x1[j] = x2[j] = 0.f;
+        if (i < half) {
+            x1[j] = to_float(row[i]);
+            x2[j] = to_float(row[i + half]);
+            ss += x1[j] * x1[j] + x2[j] * x2[j];
+        }
+    }
+    if (weight) {
+        ss = wave_sum(ss);
+        const float scale = rsqrtf(ss / (float)head_dim + eps);
+#pragma unroll
+        for (int j = 0; j < NVA_MAX_PER_LANE; ++j) {
+            const int i = lane + j * NVA_WAVE;
+            if (i < half) {
+                const float w1 = w_is_f32 ? ((const float*)weight)[i] : to_float(((const T*)weight)[i]);
+                const float w2 = w_is_f32 ? ((const float*)weight)[i + half] : to_float(((const T*)weight)[i + half]);
+                x1[j] = round_through<T>(round_through<T>(x1[j] * scale) * w1);
+                x2[j] = round_through<T>(round_through<T>(x2[j] * scale) * w2);
+            }
+        }
+    }
+    // Rotation of the pair (i, i + head_dim/2), which is exactly (x1, x2).  The table row holds
+    // head_dim/2 cosines, then head_dim/2 sines.
+    const float* angles = table ? table + (int64_t)positions[t] * head_dim : nullptr;
+    T* k_dst = nullptr;
+    if (!is_q && slot >= 0 && k_cache) {
+        const int h = head - num_q_heads;
+        const int64_t page = slot / page_size, off = slot % page_size;
+        k_dst = k_cache + ((page * num_kv_heads + h) * (int64_t)page_size + off) * head_dim;
+    }
+    if (angles) {
+#pragma unroll
+        for (int j = 0; j < NVA_MAX_PER_LANE; ++j) {
+            const int i = lane + j * NVA_WAVE;
+            if (i < half) {
+                const float c = angles[i], s = angles[half + i];
+                const float y1 = x1[j] * c - x2[j] * s;
+                const float y2 = x2[j] * c + x1[j] * s;
+                x1[j] = y1;
+                x2[j] = y2;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NVA_MAX_PER_LANE; ++j) {
+        const int i = lane + j * NVA_WAVE;
+        if (i < half) {
+            const T a = from_float<T>(x1[j]), b = from_float<T>(x2[j]);
+            row[i] = a;
+            row[i + half] = b;
+            if (k_dst) {
+                k_dst[i] = a;
+                k_dst[i + half] = b;
+            }
+        }
+    }
+}
+
+// qkv rows hold [q heads | k heads | v heads] of head_dim each.  q_weight / k_weight may be null
+// (no norm), table may be null (no rotation), the caches may be null (nothing is stored).
+// table_rows is the number of positions the table covers; positions are checked on the host.
+NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store)(void* qkv, int64_t row_stride, int64_t tokens, int num_q_heads,
+                                                int num_kv_heads, int head_dim, const void* q_weight,
+                                                const void* k_weight, int w_is_f32, float eps, const float* table,
+                                                const int32_t* positions, const int32_t* slots, void* k_cache,
+                                                void* v_cache, int page_size, hipStream_t stream) {
+    if (tokens == 0) return 0;
+    if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("qk_norm_rope_store: bad token count %lld", (long long)tokens);
+    if (num_q_heads < 0 || num_kv_heads <= 0 || head_dim <= 0)
+        return nva_fail("qk_norm_rope_store: bad heads q=%d kv=%d head_dim=%d", num_q_heads, num_kv_heads, head_dim);
+    if (head_dim % 2 || head_dim / 2 > NVA_WAVE * NVA_MAX_PER_LANE)
+        return nva_fail("qk_norm_rope_store: head_dim %d must be even and at most %d", head_dim,
+                        2 * NVA_WAVE * NVA_MAX_PER_LANE);
+    if ((k_cache || v_cache) && (page_size <= 0 || !slots))
+        return nva_fail("qk_norm_rope_store: a cache needs a page size and slots");
+    if (table && !positions) return nva_fail("qk_norm_rope_store: a rotation table needs positions");
+    const int total = num_q_heads + 2 * num_kv_heads;
+    const int waves = 4;
+    dim3 grid((unsigned)tokens, (total + waves - 1) / waves);
+    hipLaunchKernelGGL(qk_norm_rope_store_kernel<elem_t>, grid, dim3(waves * NVA_WAVE), 0, stream, (elem_t*)qkv,
+                       row_stride, num_q_heads, num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table,
+                       positions, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size);
+    return nva_check_launch("qk_norm_rope_store");
+}
+
+NVA_DEFINE_LAST_ERROR(nva_rope)

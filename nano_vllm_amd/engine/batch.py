@@ -1,0 +1,141 @@
+"""A step's batch: requests with their next tokens, flattened for the kernels.
+
+Reference: prepare_prefill / prepare_decode of nanovllm/engine/model_runner.py:129-188 and the
+Context of nanovllm/utils/context.py:5-27.  Here one description covers every mixture:
+entries with one token (decoding) come first, portions of prompts after them; each token
+carries its request's index and its absolute position, each request the number of keys it
+sees (tokens in the cache after this step) and its block table per cache group.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional, Sequence
+
+import torch
+
+
+@dataclass
+class StepEntry:
+    request: Hashable
+    tokens: Sequence[int]            # the tokens this step runs for the request
+    start: int                       # absolute position of tokens[0] = tokens already in the cache
+    want: Sequence[int] = ()         # places among `tokens` whose logits are wanted
+
+
+@dataclass
+class GroupBatch:
+    block_tables: torch.Tensor       # int32 [S, pages]; -1: no page
+    slot_mapping: torch.Tensor       # int32 [T]: page * page_size + offset of each token's key
+
+
+@dataclass
+class StepBatch:
+    num_tokens: int
+    num_seqs: int
+    num_decode: int                  # leading requests that bring exactly one token
+    input_ids: torch.Tensor          # int32 [T]
+    positions: torch.Tensor          # int32 [T] absolute positions
+    token_seq: torch.Tensor          # int32 [T] index of the token's request in this batch
+    cu_seqlens_q: torch.Tensor       # int32 [S+1]
+    kv_lens: torch.Tensor            # int32 [S] keys each request sees = start + its tokens
+    seq_starts: torch.Tensor         # int32 [S] tokens each request had in the cache before
+    state_slots: torch.Tensor        # int32 [S]
+    logits_rows: Optional[torch.Tensor]   # int32 [R] flat token indices, in the caller's order
+    groups: List[GroupBatch]
+    max_q_len: int
+    max_kv_len: int
+    # host copies
+    q_lens: List[int] = field(default_factory=list)
+    starts: List[int] = field(default_factory=list)
+    requests: List[Hashable] = field(default_factory=list)
+
+
+def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size: int, device) -> StepBatch:
+    """Orders the entries (single tokens first), checks them against the cache manager's
+    block tables and uploads everything in one copy."""
+    if not entries:
+        raise ValueError("a step needs at least one entry")
+    order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
+    offsets = {}
+    t = 0
+    for i in order:
+        offsets[i] = t
+        t += len(entries[i].tokens)
+    T, S = t, len(entries)
+    num_groups = len(cache.groups)
+
+    input_ids, positions, token_seq = [], [], []
+    cu, kv_lens, starts, state_slots, q_lens = [0], [], [], [], []
+    slot_maps = [[] for _ in range(num_groups)]
+    tables = [[] for _ in range(num_groups)]
+    seen = set()
+    for s, i in enumerate(order):
+        e = entries[i]
+        n = len(e.tokens)
+        if n == 0:
+            raise ValueError(f"request {e.request!r} brings no token")
+        if e.request in seen:
+            raise ValueError(f"request {e.request!r} appears twice in one step")
+        seen.add(e.request)
+        rc = cache.requests[e.request]
+        if e.start < 0 or e.start + n > rc.num_tokens:
+            raise ValueError(f"request {e.request!r}: positions {e.start}..{e.start + n - 1} are not reserved "
+                             f"in the cache ({rc.num_tokens} are)")
+        for tok in e.tokens:
+            if not 0 <= tok < vocab_size:
+                raise ValueError(f"request {e.request!r}: token id {tok} is outside the vocabulary of {vocab_size}")
+        input_ids.extend(e.tokens)
+        positions.extend(range(e.start, e.start + n))
+        token_seq.extend([s] * n)
+        cu.append(cu[-1] + n)
+        kv_lens.append(e.start + n)
+        starts.append(e.start)
+        q_lens.append(n)
+        state_slots.append(rc.state_slot)
+        for g in range(num_groups):
+            table = rc.tables[g]
+            tables[g].append(table)
+            sm = slot_maps[g]
+            for pos in range(e.start, e.start + n):
+                page = table[pos // page_size]
+                if page < 0:
+                    raise ValueError(f"request {e.request!r}: position {pos} has no page in group {g}")
+                sm.append(page * page_size + pos % page_size)
+    rows = []
+    for i, e in enumerate(entries):
+        for w in e.want:
+            if not 0 <= w < len(e.tokens):
+                raise ValueError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
+            rows.append(offsets[i] + w)
+
+    widths = [max(1, max(len(tb) for tb in tables[g])) for g in range(num_groups)]
+    flat: List[int] = []
+    flat += input_ids + positions + token_seq + cu + kv_lens + starts + state_slots + rows
+    for g in range(num_groups):
+        flat += slot_maps[g]
+        for tb in tables[g]:
+            flat += tb + [-1] * (widths[g] - len(tb))
+    dev = torch.tensor(flat, dtype=torch.int32).to(device)
+
+    pos = 0
+
+    def take(n):
+        nonlocal pos
+        out = dev[pos:pos + n]
+        pos += n
+        return out
+
+    b_ids, b_pos, b_seq = take(T), take(T), take(T)
+    b_cu, b_kv, b_starts, b_slots = take(S + 1), take(S), take(S), take(S)
+    b_rows = take(len(rows)) if rows else None
+    groups = []
+    for g in range(num_groups):
+        sm = take(T)
+        bt = take(S * widths[g]).view(S, widths[g])
+        groups.append(GroupBatch(bt, sm))
+    return StepBatch(
+        num_tokens=T, num_seqs=S, num_decode=sum(1 for n in q_lens if n == 1),
+        input_ids=b_ids, positions=b_pos, token_seq=b_seq, cu_seqlens_q=b_cu, kv_lens=b_kv,
+        seq_starts=b_starts, state_slots=b_slots, logits_rows=b_rows, groups=groups,
+        max_q_len=max(q_lens), max_kv_len=max(kv_lens), q_lens=q_lens, starts=starts,
+        requests=[entries[i].request for i in order])

@@ -1,0 +1,74 @@
+"""The model runner: owns the model, the cache tensors and the step function.
+
+Reference: nanovllm/engine/model_runner.py - ModelRunner.run (:214-220) with its
+prepare_* helpers, allocate_kv_cache (:103-121).  One step function serves every caller
+(the engine loop and the trace replay): it runs exactly the tokens it is given, as one
+batch, from the cache, and returns float32 logits at the wanted places.  Sampling is a
+separate call.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import torch
+
+from ..cache.manager import CacheManager, plan_groups
+from ..cache import storage
+from ..config.model_config import read_config_json
+from ..config.registry import architecture_of
+from ..kernels import HipKernels
+from ..parts.model import Model, torch_dtype
+from ..weights.loader import load_weights
+from .batch import StepBatch, StepEntry, build_batch
+
+
+class ModelRunner:
+    def __init__(self, model: Model, page_size: int, num_pages, max_requests: int,
+                 enable_prefix_caching: bool = True):
+        """num_pages: pages per cache group (an int for every group, or one per group)."""
+        self.model = model
+        self.kernels = model.kernels
+        self.device = model.device
+        self.page_size = page_size
+        self.needs = model.cache_needs()
+        self.groups, self.state_runs = plan_groups(self.needs)
+        counts = list(num_pages) if isinstance(num_pages, (list, tuple)) else [num_pages] * len(self.groups)
+        self.cache = CacheManager(self.groups, page_size, counts,
+                                  num_state_slots=max_requests if self.state_runs else 0,
+                                  has_state=bool(self.state_runs), enable_prefix_caching=enable_prefix_caching)
+        self.layer_caches = storage.allocate(self.needs, self.groups, self.state_runs, counts, page_size,
+                                             max_requests, model.dtype, self.device)
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_folder(cls, folder: str, dtype: Optional[str] = None, device="cuda:0", page_size: int = 256,
+                    num_pages=None, max_requests: int = 512, kernels=None, quiet: bool = False,
+                    enable_prefix_caching: bool = True) -> "ModelRunner":
+        model = load_model(folder, dtype, device, kernels, quiet)
+        return cls(model, page_size, num_pages, max_requests, enable_prefix_caching)
+
+    # ------------------------------------------------------------------ the step
+    @torch.inference_mode()
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Runs the entries' tokens as one batch.  Their pages must be reserved in
+        self.cache.  Returns float32 logits [wanted places, vocab] in the order of the
+        entries and of their `want`, or None if nothing is wanted."""
+        batch = build_batch(entries, self.cache, self.page_size, self.model.spec.vocab_size, self.device)
+        hidden = self.model.forward(batch, self.layer_caches)
+        if batch.logits_rows is None:
+            return None
+        return self.model.logits(hidden, batch.logits_rows)
+
+
+def load_model(folder: str, dtype: Optional[str] = None, device="cuda:0", kernels=None, quiet: bool = False) -> Model:
+    """config.json -> architecture -> ModelSpec -> Model, then the weights of the folder."""
+    config_json = read_config_json(folder)
+    arch = architecture_of(config_json)
+    config = arch.parse_config(config_json)
+    spec = arch.build_spec(config)
+    tdtype = torch_dtype(dtype or spec.dtype)
+    if kernels is None:
+        kernels = HipKernels(device, tdtype, quiet=quiet)        # raises without a GPU or the compiled kernels
+    model = Model(spec, kernels, device, tdtype)
+    load_weights(model, folder)
+    return model

@@ -1,0 +1,290 @@
+"""The operations the parts call, bound to the HIP kernels under csrc/.
+
+Each method checks on the host that operand shapes, strides and types match what its
+kernel and grid assume, then launches on torch's current stream.  torch is the allocator
+and stream owner; the only library computation left is the bfloat16 matrix product for
+many rows, where the reference uses a library as well (nanovllm/layers/linear.py:51,73,153).
+
+Cache layouts (chosen for the attention kernels):
+    K [pages, kv_heads, page_size, head_dim]
+    V [pages, kv_heads, head_dim, page_size]      (transposed: keys are contiguous)
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import library
+from .library import KernelError
+
+_SUFFIX = {torch.bfloat16: "bf16", torch.float32: "f32"}
+
+c_i32, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else c_ptr(t.data_ptr())
+
+
+def _suffix(t: torch.Tensor) -> str:
+    try:
+        return _SUFFIX[t.dtype]
+    except KeyError:
+        raise KernelError(f"no kernels for element type {t.dtype}; bfloat16 and float32 are built") from None
+
+
+def _rows2d(t: torch.Tensor, what: str) -> Tuple[int, int, int]:
+    """(rows, width, row stride) of a 2-D tensor whose rows are contiguous."""
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{what}: expected a 2-D tensor with contiguous rows, got shape "
+                          f"{tuple(t.shape)} strides {t.stride()}")
+    return t.shape[0], t.shape[1], t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _i32(t: torch.Tensor, n: int, what: str):
+    if t.dtype != torch.int32 or t.dim() != 1 or t.shape[0] != n or not t.is_contiguous():
+        raise KernelError(f"{what}: expected contiguous int32[{n}], got {t.dtype}{tuple(t.shape)}")
+
+
+class HipKernels:
+    """Every device operation of the engine.  Needs a GPU and the compiled libraries."""
+
+    name = "hip"
+
+    def __init__(self, device="cuda:0", dtype: torch.dtype = torch.bfloat16, quiet: bool = False):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: the engine runs on HIP kernels only and has no CPU path")
+        if dtype not in _SUFFIX:
+            raise KernelError(f"no kernels for element type {dtype}; bfloat16 and float32 are built")
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.suffix = _SUFFIX[dtype]
+        library.preload(self.suffix, quiet=quiet)       # compiles what this element type needs
+        # bit 0: a token id outside the vocabulary; bit 1: a visible key without a page
+        self.fault_flag = torch.zeros(1, dtype=torch.int32, device=self.device)
+        # Rows up to which the bfloat16 product runs on the engine's own kernels.
+        self.own_matmul_rows = 0
+
+    # ------------------------------------------------------------------ helpers
+    def _stream(self):
+        return c_ptr(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def check_faults(self) -> None:
+        """Reads the device-side fault flags (a synchronising copy) and raises on any."""
+        flags = int(self.fault_flag.item())
+        if flags:
+            self.fault_flag.zero_()
+            what = []
+            if flags & 1:
+                what.append("a token id outside the vocabulary reached the embedding")
+            if flags & 2:
+                what.append("attention met a visible key whose page is missing from the block table")
+            raise KernelError("device-side check failed: " + "; ".join(what))
+
+    # ------------------------------------------------------------------ rows
+    def embedding(self, table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """out[t] = table[ids[t]]; also used to pick rows of activations."""
+        rows, width, stride = _rows2d(table, "embedding table")
+        n = ids.shape[0]
+        _i32(ids, n, "embedding ids")
+        if out is None:
+            out = torch.empty((n, width), dtype=table.dtype, device=table.device)
+        _, ow, ostride = _rows2d(out, "embedding out")
+        if ow != width or out.dtype != table.dtype or out.shape[0] != n:
+            raise KernelError("embedding: output does not match the table")
+        library.call("embed", _suffix(table), "nva_gather_rows", _p(table), c_i64(stride), c_i64(rows), _p(ids),
+                     _p(out), c_i64(ostride), c_i64(n), c_i32(width), _p(self.fault_flag), self._stream())
+        return out
+
+    gather_rows = embedding
+
+    # ------------------------------------------------------------------ norms
+    def _norm_weight(self, weight: torch.Tensor, width: int, x: torch.Tensor):
+        if weight.dim() != 1 or weight.shape[0] != width or not weight.is_contiguous():
+            raise KernelError(f"norm weight must be contiguous [{width}], got {tuple(weight.shape)}")
+        if weight.dtype == torch.float32:
+            return 1
+        if weight.dtype != x.dtype:
+            raise KernelError(f"norm weight is {weight.dtype}; expected float32 or the input's {x.dtype}")
+        return 0
+
+    def rms_norm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None):
+        rows, width, xs = _rows2d(x, "rms_norm input")
+        wf = self._norm_weight(weight, width, x)
+        if out is None:
+            out = torch.empty((rows, width), dtype=x.dtype, device=x.device)
+        orows, ow, os_ = _rows2d(out, "rms_norm output")
+        if (orows, ow) != (rows, width) or out.dtype != x.dtype:
+            raise KernelError("rms_norm: output does not match the input")
+        library.call("norm", _suffix(x), "nva_rms_norm", _p(x), c_i64(xs), _p(weight), c_i32(wf), _p(out),
+                     c_i64(os_), c_i64(rows), c_i32(width), c_f32(eps), self._stream())
+        return out
+
+    def add_rms_norm(self, x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float,
+                     out: Optional[torch.Tensor] = None):
+        """residual <- x + residual (in place); returns (norm(residual) * weight, residual)."""
+        rows, width, xs = _rows2d(x, "add_rms_norm input")
+        rrows, rw, rs = _rows2d(residual, "add_rms_norm residual")
+        if (rrows, rw) != (rows, width) or residual.dtype != x.dtype:
+            raise KernelError("add_rms_norm: residual does not match the input")
+        wf = self._norm_weight(weight, width, x)
+        if out is None:
+            out = torch.empty((rows, width), dtype=x.dtype, device=x.device)
+        orows, ow, os_ = _rows2d(out, "add_rms_norm output")
+        if (orows, ow) != (rows, width) or out.dtype != x.dtype:
+            raise KernelError("add_rms_norm: output does not match the input")
+        library.call("norm", _suffix(x), "nva_add_rms_norm", _p(x), c_i64(xs), _p(residual), c_i64(rs), _p(weight),
+                     c_i32(wf), _p(out), c_i64(os_), c_i64(rows), c_i32(width), c_f32(eps), self._stream())
+        return out, residual
+
+    # ------------------------------------------------------------------ feed-forward
+    def silu_mul(self, gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        rows, width, xs = _rows2d(gate_up, "silu_mul input")
+        if width % 2:
+            raise KernelError("silu_mul: the input holds gate and up halves, its width must be even")
+        inner = width // 2
+        if out is None:
+            out = torch.empty((rows, inner), dtype=gate_up.dtype, device=gate_up.device)
+        orows, ow, os_ = _rows2d(out, "silu_mul output")
+        if (orows, ow) != (rows, inner) or out.dtype != gate_up.dtype:
+            raise KernelError("silu_mul: output does not match the input")
+        library.call("activation", _suffix(gate_up), "nva_silu_mul", _p(gate_up), c_i64(xs), _p(out), c_i64(os_),
+                     c_i64(rows), c_i32(inner), self._stream())
+        return out
+
+    # ------------------------------------------------------------------ matrix products
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               out_float32: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """y = x @ weight.T (+ bias), weight [out, in].  float32 inputs run the engine's own
+        float kernel; bfloat16 inputs with many rows run the library product."""
+        m, k, xs = _rows2d(x, "linear input")
+        n, wk, ws = _rows2d(weight, "linear weight")
+        if wk != k or weight.dtype != x.dtype:
+            raise KernelError(f"linear: input [{m},{k}] {x.dtype} does not fit weight [{n},{wk}] {weight.dtype}")
+        if bias is not None and (bias.shape != (n,) or bias.dtype != x.dtype or not bias.is_contiguous()):
+            raise KernelError("linear: bias does not fit")
+        out_dtype = torch.float32 if out_float32 else x.dtype
+        if x.dtype == torch.bfloat16 and not out_float32 and m > self.own_matmul_rows:
+            y = torch.nn.functional.linear(x, weight, bias)
+            if out is not None:
+                out.copy_(y)
+                return out
+            return y
+        if out is None:
+            out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+        om, on, os_ = _rows2d(out, "linear output")
+        if (om, on) != (m, n) or out.dtype != out_dtype:
+            raise KernelError("linear: output does not match")
+        library.call("gemm", _suffix(x), "nva_linear_tiled", _p(x), c_i64(xs), _p(weight), c_i64(ws), _p(bias),
+                     _p(out), c_i64(os_), c_i32(1 if out_dtype == torch.float32 and x.dtype != torch.float32 else 0),
+                     c_i64(m), c_i64(n), c_i64(k), self._stream())
+        return out
+
+    def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+        """silu(x @ Wg.T) * (x @ Wu.T) with weight = [Wg; Wu]."""
+        return self.silu_mul(self.linear(x, weight))
+
+    # ------------------------------------------------------------------ position encoding
+    def rotary_table(self, inv_freq: torch.Tensor, num_positions: int) -> torch.Tensor:
+        """float32 [positions, 2 * len(inv_freq)]: cos(p * f) then sin(p * f)."""
+        if inv_freq.dtype != torch.float32 or inv_freq.dim() != 1 or not inv_freq.is_contiguous():
+            raise KernelError("rotary_table: inv_freq must be contiguous float32")
+        half = inv_freq.shape[0]
+        table = torch.empty((num_positions, 2 * half), dtype=torch.float32, device=inv_freq.device)
+        library.call("rope", self.suffix, "nva_rotary_table", _p(inv_freq), c_i32(half), c_i64(num_positions), _p(table),
+                     self._stream())
+        return table
+
+    def qk_norm_rope_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                           q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                           table: Optional[torch.Tensor], positions: Optional[torch.Tensor],
+                           slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                           v_cache: Optional[torch.Tensor]) -> torch.Tensor:
+        """Per-head norm of q and k, rotation by the table's rows, q and k written back in
+        place, k and v written into their page slots.  Returns the q view [T, heads*head_dim]."""
+        tokens, width, stride = _rows2d(qkv, "qkv")
+        if width != (num_heads + 2 * num_kv_heads) * head_dim:
+            raise KernelError(f"qkv width {width} is not (heads + 2*kv_heads) * head_dim = "
+                              f"{(num_heads + 2 * num_kv_heads) * head_dim}")
+        wf = 0
+        for w in (q_weight, k_weight):
+            if w is not None:
+                wf = self._norm_weight(w, head_dim, qkv)
+        if (q_weight is None) != (k_weight is None):
+            raise KernelError("qk norm: give both weights or none")
+        if q_weight is not None and q_weight.dtype != k_weight.dtype:
+            raise KernelError("qk norm: the two weights differ in type")
+        if table is not None:
+            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != head_dim or not table.is_contiguous():
+                raise KernelError(f"rotary table must be float32 [positions, {head_dim}]: partial rotation is not built")
+            _i32(positions, tokens, "positions")
+        page_size = 0
+        if k_cache is not None:
+            page_size = self._check_cache(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype)
+            _i32(slots, tokens, "slots")
+        library.call("rope", _suffix(qkv), "nva_qk_norm_rope_store", _p(qkv), c_i64(stride), c_i64(tokens),
+                     c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim), _p(q_weight), _p(k_weight), c_i32(wf),
+                     c_f32(eps), _p(table), _p(positions), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size),
+                     self._stream())
+        return qkv[:, : num_heads * head_dim]
+
+    @staticmethod
+    def _check_cache(k_cache, v_cache, num_kv_heads, head_dim, dtype) -> int:
+        if k_cache.dim() != 4 or v_cache is None or v_cache.dim() != 4:
+            raise KernelError("cache tensors must be K [pages, kv_heads, page, head_dim] and V [pages, kv_heads, head_dim, page]")
+        pages, h, page_size, d = k_cache.shape
+        if (h, d) != (num_kv_heads, head_dim) or tuple(v_cache.shape) != (pages, h, d, page_size):
+            raise KernelError(f"cache shapes K {tuple(k_cache.shape)} V {tuple(v_cache.shape)} do not fit "
+                              f"{num_kv_heads} kv heads of {head_dim}")
+        if not (k_cache.is_contiguous() and v_cache.is_contiguous()) or k_cache.dtype != dtype or v_cache.dtype != dtype:
+            raise KernelError("cache tensors must be contiguous and of the activations' type")
+        return page_size
+
+    # ------------------------------------------------------------------ attention
+    def paged_attention(self, q: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                        k_cache: torch.Tensor, v_cache: torch.Tensor, batch, group: int, scale: float,
+                        window: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Causal attention of the step's tokens over the cache.  `batch` is the step's
+        StepBatch; `group` selects its block tables.  q [T, heads*head_dim] (rows may be strided)."""
+        tokens, width, qs = _rows2d(q, "attention q")
+        if width != num_heads * head_dim:
+            raise KernelError("attention: q width is not heads * head_dim")
+        page_size = self._check_cache(k_cache, v_cache, num_kv_heads, head_dim, q.dtype)
+        if num_heads % num_kv_heads:
+            raise KernelError(f"attention: {num_heads} heads do not divide into {num_kv_heads} kv heads")
+        tables = batch.groups[group].block_tables
+        if tables.dtype != torch.int32 or tables.dim() != 2 or tables.shape[0] != batch.num_seqs or not tables.is_contiguous():
+            raise KernelError("attention: block tables must be contiguous int32 [requests, pages]")
+        _i32(batch.token_seq, tokens, "token_seq")
+        _i32(batch.positions, tokens, "positions")
+        need_pages = (batch.max_kv_len + page_size - 1) // page_size
+        if tables.shape[1] < need_pages:
+            raise KernelError(f"attention: block tables hold {tables.shape[1]} pages, {need_pages} are needed")
+        if out is None:
+            out = torch.empty((tokens, width), dtype=q.dtype, device=q.device)
+        _, ow, os_ = _rows2d(out, "attention out")
+        if ow != width or out.shape[0] != tokens or out.dtype != q.dtype:
+            raise KernelError("attention: output does not match q")
+        library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q), c_i64(qs), _p(out), c_i64(os_),
+                     _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.token_seq),
+                     _p(batch.positions), c_i64(tokens), c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim),
+                     c_i32(page_size), c_f32(scale), c_i32(window or 0), _p(self.fault_flag), self._stream())
+        return out
+
+    # ------------------------------------------------------------------ sampling
+    def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:
+        """int32 [rows]: argmax where temperature is 0, else a draw from softmax(logits / T)
+        with the row's counter-based noise key (int64 bit pattern of a 64-bit key)."""
+        rows, vocab, stride = _rows2d(logits, "logits")
+        if logits.dtype != torch.float32:
+            raise KernelError("sample: logits must be float32")
+        if temperatures.dtype != torch.float32 or temperatures.shape != (rows,) or not temperatures.is_contiguous():
+            raise KernelError("sample: temperatures must be float32 [rows]")
+        if keys.dtype != torch.int64 or keys.shape != (rows,) or not keys.is_contiguous():
+            raise KernelError("sample: keys must be int64 [rows]")
+        out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        library.call("sample", None, "nva_sample", _p(logits), c_i64(stride), c_i64(rows), c_i32(vocab),
+                     _p(temperatures), _p(keys), _p(out), self._stream())
+        return out

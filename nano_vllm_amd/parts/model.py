@@ -1,0 +1,143 @@
+"""The model: parts put together as a ModelSpec says.
+
+Reference for the whole: nanovllm/models/qwen3.py:162-216 (embedding, the layers in order,
+final norm, output head with optionally tied embedding).  Here the layers and their order
+are data: Model knows no architecture.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Mapping, Optional, Tuple
+
+import torch
+
+from .base import BuildContext, ParamDecl, Part, named_params
+from .registry import make_part
+from .spec import LayerRun, ModelSpec, PartSpec
+
+_TORCH_DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+
+
+def torch_dtype(name: str) -> torch.dtype:
+    try:
+        return _TORCH_DTYPES[name]
+    except KeyError:
+        raise ValueError(f"element type {name!r} has no kernels: use bfloat16 or float32") from None
+
+
+@dataclass
+class LayerCache:
+    """What one run of the order owns in the cache: the index of its page group in the
+    step's batch and its tensors there, or its per-request state tensors [slots, ...]."""
+    group: int = -1
+    k: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None
+    state: Optional[Dict[str, torch.Tensor]] = None
+
+
+class TokenEmbedding(Part):
+    """weight [vocab, hidden]; rows are gathered by token id (embed_head.py:24,38)."""
+
+    def __init__(self, params: Mapping, build: BuildContext):
+        super().__init__(params, build)
+        self.vocab, self.hidden = int(params["vocab_size"]), int(params["hidden_size"])
+
+    def param_decls(self):
+        return {"weight": ParamDecl((self.vocab, self.hidden))}
+
+    def forward(self, ids):
+        return self.kernels.embedding(self.weights["weight"], ids)
+
+
+class OutputHead(Part):
+    """logits = x W^T in float32, W [vocab, hidden] (embed_head.py:61); tied: W is the
+    embedding's storage and the checkpoint holds no tensor for it (qwen3.py:202-203)."""
+
+    def __init__(self, params: Mapping, build: BuildContext):
+        super().__init__(params, build)
+        self.vocab, self.hidden = int(params["vocab_size"]), int(params["hidden_size"])
+        self.tied = bool(params.get("tied", False))
+
+    def param_decls(self):
+        return {} if self.tied else {"weight": ParamDecl((self.vocab, self.hidden))}
+
+    def forward(self, x):
+        return self.kernels.linear(x, self.weights["weight"], out_float32=True)
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, kernels, device="cuda:0", dtype: Optional[torch.dtype] = None):
+        spec.validate()
+        self.spec = spec
+        self.kernels = kernels
+        self.device = torch.device(device)
+        self.dtype = dtype or torch_dtype(spec.dtype)
+        build = BuildContext(kernels, self.device, self.dtype, spec.hidden_size, spec.max_position)
+        for name, pe in spec.position_encodings.items():
+            build.position_encodings[name] = make_part("position_encoding", pe, build)
+        self.position_encodings = build.position_encodings
+        sizes = {"vocab_size": spec.vocab_size, "hidden_size": spec.hidden_size}
+        self.embedding = TokenEmbedding({**spec.embedding.params, **sizes}, build)
+        self.blocks: List[Part] = []
+        for layer in spec.layers:
+            block_spec = PartSpec(layer.block.kind, {**layer.block.params, "parts": layer.parts, "names": layer.names})
+            self.blocks.append(make_part("block", block_spec, build))
+        self.final_norm = make_part("norm", spec.final_norm, build)
+        self.head = OutputHead({**spec.head.params, **sizes}, build)
+        self.order: Tuple[LayerRun, ...] = spec.order
+
+        # full parameter name -> (owner part, local name, declaration)
+        self.param_table: Dict[str, Tuple[Part, str, ParamDecl]] = {}
+        roots = [(spec.embedding["name"], self.embedding), (spec.final_norm["name"], self.final_norm),
+                 (spec.head["name"], self.head)]
+        roots += [(layer.name, block) for layer, block in zip(spec.layers, self.blocks)]
+        for prefix, part in roots:
+            for full, owner, local, decl in named_params(part, prefix):
+                if full in self.param_table:
+                    raise ValueError(f"two parts declare the parameter {full!r}")
+                self.param_table[full] = (owner, local, decl)
+        self.params: Dict[str, torch.Tensor] = {}
+
+    # ------------------------------------------------------------------ weights
+    def set_param(self, name: str, tensor: torch.Tensor) -> None:
+        owner, local, decl = self.param_table[name]
+        if tuple(tensor.shape) != tuple(decl.shape):
+            raise ValueError(f"parameter {name}: shape {tuple(tensor.shape)} is not {tuple(decl.shape)}")
+        self.params[name] = tensor
+        owner.weights[local] = tensor
+
+    def finish_weights(self) -> None:
+        missing = [n for n in self.param_table if n not in self.params]
+        if missing:
+            raise ValueError(f"parameters without a tensor: {missing}")
+        if self.head.tied:
+            self.head.weights["weight"] = self.embedding.weights["weight"]
+
+    def num_parameters(self) -> int:
+        return sum(int(torch.tensor(d.shape).prod()) for _, _, d in self.param_table.values())
+
+    # ------------------------------------------------------------------ cache
+    def cache_needs(self):
+        """Per entry of the order: what its cache must hold, or None when it reads another's."""
+        return [self.blocks[run.layer].cache_need() if run.cache_of is None else None for run in self.order]
+
+    def cache_owner(self, i: int) -> int:
+        run = self.order[i]
+        return i if run.cache_of is None else run.cache_of
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, batch, caches: List[LayerCache]) -> torch.Tensor:
+        """Hidden states [T, hidden] of the batch's tokens after the final norm."""
+        h = self.embedding.forward(batch.input_ids)
+        residual = None
+        for i, run in enumerate(self.order):
+            h, residual = self.blocks[run.layer].forward(h, residual, batch, caches[self.cache_owner(i)])
+        if residual is None:
+            return self.final_norm.forward(h)
+        h, _ = self.final_norm.forward_add(h, residual)
+        return h
+
+    def logits(self, hidden: torch.Tensor, rows: Optional[torch.Tensor]) -> torch.Tensor:
+        """float32 [R, vocab] at the given flat token indices (all tokens if None)."""
+        x = hidden if rows is None else self.kernels.gather_rows(hidden, rows)
+        return self.head.forward(x)
