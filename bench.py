@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+The default run has the layer sizes of the Qwen3-8B shape (36 layers, hidden 4096, 32 query
+and 8 kv heads of 128, inner 12288, vocabulary 151936, bfloat16) with seeded random weights,
+a batch of 8 requests and a context of 4096 tokens: after W untimed steps, K decode steps
+(one token per request and step, through the engine's step function and sampler) are timed
+so that the last one ends at the context length.  The cache in front of the timed steps is
+filled with random keys and values (a decode step's work does not depend on their values).
+Also measured: a prefill of 2,048 tokens, and decoding at batch 1 and 64.
+
+One JSON line is printed: `value` is decoded tokens a second at the default batch.
+The reference measures throughput the same way on synthetic token ids (bench.py:8-28 there).
+"""
+import argparse
+import json
+import sys
+import time
+
+PEAK_HBM_GBS = 8000.0                      # MI355X HBM3E, published
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float32": 157.3e12}      # dense MFMA, published
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=36, help="layers to build (the shape has 36)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--page-size", type=int, default=256)
+    ap.add_argument("--points", default="1,64", help="further decode batch sizes")
+    ap.add_argument("--eager", action="store_true", help="no captured decode graph")
+    ap.add_argument("--seed", type=int, default=0)
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not measured")
+        return 2
+
+    import torch
+    from nano_vllm_amd.config import Qwen3Config
+    from nano_vllm_amd.engine.batch import StepEntry
+    from nano_vllm_amd.engine.runner import ModelRunner
+    from nano_vllm_amd.kernels import HipKernels
+    from nano_vllm_amd.models.qwen3 import build_spec
+    from nano_vllm_amd.parts.model import Model, torch_dtype
+    from nano_vllm_amd.sampling.sampler import Sampler
+    from nano_vllm_amd.weights import fill_random_
+
+    full_layers = 36
+    cfg = Qwen3Config(vocab_size=151936, hidden_size=4096, num_hidden_layers=args.layers, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, intermediate_size=12288, rms_norm_eps=1e-6,
+                      rope_theta=1000000.0, max_position_embeddings=40960, tie_word_embeddings=False,
+                      dtype=args.dtype)
+    device = "cuda:0"
+    dtype = torch_dtype(args.dtype)
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    kernels = HipKernels(device, dtype)
+    model = Model(build_spec(cfg), kernels, device, dtype)
+    fill_random_(model, args.seed)
+    torch.cuda.synchronize()
+
+    points = sorted({args.batch} | {int(b) for b in args.points.split(",") if b})
+    page = args.page_size
+    pages_per_request = (args.context + page - 1) // page + 1
+    num_pages = max(points) * pages_per_request + (args.prefill_tokens + page - 1) // page + 1
+    runner = ModelRunner(model, page, num_pages, max(points) + 1, enable_prefix_caching=False)
+    if not args.eager and hasattr(runner, "enable_decode_graphs"):
+        runner.enable_decode_graphs(max(points), args.context + page)
+    for lc in runner.layer_caches:                      # random keys and values in every page
+        lc.k.normal_(0, 1)
+        lc.v.normal_(0, 1)
+    sampler = Sampler(kernels, model.device)
+    gen = torch.Generator().manual_seed(args.seed)
+
+    # ------------------------------------------------------------------ what a decode step must read
+    H, I, V, D = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.head_dim
+    Hq, Hkv, L = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.num_hidden_layers
+    layer_matrix_params = (Hq + 2 * Hkv) * D * H + H * Hq * D + 2 * I * H + H * I
+    layer_params = layer_matrix_params + 2 * H + 2 * D
+    weight_bytes = (L * layer_params + H + V * H) * itemsize            # every weight a step uses, once
+    kv_bytes_per_token = 2 * L * Hkv * D * itemsize
+
+    def decode_run(batch, steps, warmup):
+        """Timed decode steps that end with `context` tokens in each request's cache."""
+        start = args.context - (steps + warmup)
+        ids = [f"d{batch}-{i}" for i in range(batch)]
+        for rid in ids:
+            runner.cache.admit(rid)
+            runner.cache.reserve(rid, start)
+        tokens = torch.randint(0, V, (batch,), generator=gen).tolist()
+        pos = start
+        temps, seeds, reqs = [0.0] * batch, [0] * batch, list(range(batch))
+
+        def one_step():
+            nonlocal tokens, pos
+            entries = []
+            for rid, tok in zip(ids, tokens):
+                runner.cache.reserve(rid, pos + 1)
+                entries.append(StepEntry(rid, [tok], pos, [0]))
+            logits = runner.step(entries)
+            tokens = sampler.sample(logits, temps, seeds, reqs, [pos + 1] * batch)
+            pos += 1
+
+        for _ in range(warmup):
+            one_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one_step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert pos == args.context
+        for rid in ids:
+            runner.cache.release(rid)
+        # keys read per step: the mean context over the timed steps
+        mean_ctx = args.context - (steps - 1) / 2.0
+        step_bytes = weight_bytes + batch * H * itemsize + batch * mean_ctx * kv_bytes_per_token
+        return dt, step_bytes
+
+    def prefill_run(tokens_n, reps, warmup):
+        toks = torch.randint(0, V, (tokens_n,), generator=gen).tolist()
+        times = []
+        for r in range(warmup + reps):
+            runner.cache.admit("p")
+            runner.cache.reserve("p", tokens_n)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            runner.step([StepEntry("p", toks, 0, [tokens_n - 1])])
+            torch.cuda.synchronize()
+            if r >= warmup:
+                times.append(time.perf_counter() - t0)
+            runner.cache.release("p")
+        return sum(times) / len(times)
+
+    results = {}
+    for b in points:
+        steps = args.steps if b == args.batch else max(8, args.steps // 2)
+        dt, step_bytes = decode_run(b, steps, args.warmup)
+        results[b] = (b * steps / dt, dt / steps, step_bytes)
+        print(f"# decode batch {b}: {results[b][0]:.1f} tok/s, {results[b][1] * 1e3:.3f} ms/step", file=sys.stderr,
+              flush=True)
+
+    T = args.prefill_tokens
+    pre_s = prefill_run(T, reps=3, warmup=2)
+    # matrix products of every token, the head for the one wanted row, causal attention
+    prefill_flops = 2.0 * T * L * layer_matrix_params + 2.0 * V * H + L * 4.0 * Hq * D * T * (T + 1) / 2.0
+    print(f"# prefill {T} tokens: {T / pre_s:.0f} tok/s, {pre_s * 1e3:.2f} ms", file=sys.stderr, flush=True)
+    kernels.check_faults()
+
+    value, step_s, step_bytes = results[args.batch]
+    achieved = step_bytes / step_s / 1e9
+    line = {
+        "metric": "decode tok/s @ batch 8, context 4096, Qwen3-8B shape bf16 (also batch 1/64 and prefill tok/s @ 2048 tok)",
+        "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": "Qwen3-8B shape, random weights", "global_batch": args.batch, "seq_len": args.context,
+                   "parallelism": "single GPU", "layers": L, "layers_of_shape": full_layers, "hidden_size": H,
+                   "num_attention_heads": Hq, "num_key_value_heads": Hkv, "head_dim": D, "intermediate_size": I,
+                   "vocab_size": V, "kv_page_size": page, "prefill_tokens": T, "rope_theta": cfg.rope_theta,
+                   "rms_norm_eps": cfg.rms_norm_eps, "decode_graph": bool(not args.eager and hasattr(runner, "enable_decode_graphs"))},
+        "prefill": {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
+                    "frac": round(prefill_flops / pre_s / PEAK_FLOPS[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4)},
+        "points": {f"decode_b{b}": round(results[b][0], 2) for b in points if b != args.batch},
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

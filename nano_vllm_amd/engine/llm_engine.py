@@ -1,2 +1,188 @@
+"""The engine loop and the Python entry point's methods.
+
+Reference: nanovllm/engine/llm_engine.py:15-90 - LLMEngine(model, **config), add_request,
+step, is_finished, generate - with the same names and meanings.  Differences: unknown
+keyword arguments are an error instead of being dropped; prompts of token ids need no
+tokenizer, and "text" is None where none is available; temperature 0 is greedy.
+"""
+from __future__ import annotations
+
+import os
+import sys
+from time import perf_counter
+from typing import Dict, List, Optional, Sequence as Seq, Tuple, Union
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..config.model_config import read_config_json
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler
+from .batch import StepEntry
+from .runner import ModelRunner, load_model
+from .scheduler import Scheduler
+from .sequence import Sequence
+
+
 class LLMEngine:
-    pass
+    def __init__(self, model: str, kernels=None, **kwargs):
+        """kernels: None for the HIP kernels (the only implementation in the package), or an
+        object with the same operations, which tests use to run the host logic elsewhere."""
+        unknown = set(kwargs) - EngineConfig.field_names()
+        if unknown:
+            raise TypeError(f"unknown engine options {sorted(unknown)}; known: {sorted(EngineConfig.field_names())}")
+        self.config = cfg = EngineConfig(model, **kwargs)
+        self.model = load_model(cfg.model, cfg.dtype, cfg.device, kernels)
+        spec = self.model.spec
+        cfg.max_model_len = min(cfg.max_model_len, spec.max_position)           # config.py:25
+        num_pages = cfg.num_kvcache_blocks
+        if num_pages is None or num_pages <= 0:
+            num_pages = self._pages_from_free_memory()
+            cfg.num_kvcache_blocks = num_pages
+        self.runner = ModelRunner(self.model, cfg.kvcache_block_size, num_pages, cfg.max_num_seqs,
+                                  enable_prefix_caching=cfg.enable_prefix_caching)
+        eos = [cfg.eos] if cfg.eos >= 0 else list(spec.eos_token_ids) or self._eos_from_generation_config()
+        self.tokenizer = None
+        self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens,
+                                   cfg.max_model_len, eos, cfg.schedule)
+        self.sampler = Sampler(self.model.kernels, self.model.device)
+        self.stats = {"prefill_tokens": 0, "prefill_time": 0.0, "decode_tokens": 0, "decode_time": 0.0, "steps": 0}
+        self._by_id: Dict[int, Sequence] = {}
+
+    # ------------------------------------------------------------------ set-up helpers
+    def _pages_from_free_memory(self) -> int:
+        """As nanovllm/engine/model_runner.py:103-114: what gpu_memory_utilization of the
+        device leaves after the weights and a step's activations, in pages of all layers."""
+        from ..cache import storage
+        from ..cache.manager import plan_groups
+        cfg, model = self.config, self.model
+        needs = model.cache_needs()
+        groups, _ = plan_groups(needs)
+        itemsize = torch.empty((), dtype=model.dtype).element_size()
+        per_page = sum(storage.bytes_per_page(needs, groups, cfg.kvcache_block_size, itemsize))
+        if model.device.type != "cuda":
+            raise RuntimeError("num_kvcache_blocks must be given when the model is not on a GPU")
+        free, total = torch.cuda.mem_get_info(model.device)
+        used = total - free
+        # activations of the largest step: a few rows of the widest intermediate per token
+        widest = max([model.spec.hidden_size] + [d.shape[0] for _, _, d in model.param_table.values()
+                                                  if len(d.shape) == 2 and d.shape[0] < model.spec.vocab_size])
+        activations = cfg.max_num_batched_tokens * (4 * widest + 8 * model.spec.hidden_size) * itemsize
+        activations += cfg.max_num_seqs * model.spec.vocab_size * 4 * 2
+        budget = int(total * cfg.gpu_memory_utilization) - used - activations
+        pages = budget // max(per_page, 1)
+        if pages <= 0:
+            raise RuntimeError("no device memory is left for the cache (model_runner.py:114)")
+        return int(pages)
+
+    def _eos_from_generation_config(self) -> List[int]:
+        path = os.path.join(self.config.model, "generation_config.json")
+        if os.path.isfile(path):
+            import json
+            with open(path) as f:
+                eos = json.load(f).get("eos_token_id")
+            if isinstance(eos, int):
+                return [eos]
+            if isinstance(eos, list):
+                return [int(e) for e in eos]
+        return []
+
+    def _tokenizer(self):
+        if self.tokenizer is None:
+            try:
+                from transformers import AutoTokenizer      # llm_engine.py:32
+                self.tokenizer = AutoTokenizer.from_pretrained(self.config.model, use_fast=True)
+            except Exception as e:
+                raise RuntimeError(f"a text prompt needs a tokenizer in {self.config.model!r}: {e}") from e
+        return self.tokenizer
+
+    # ------------------------------------------------------------------ the reference's methods
+    def add_request(self, prompt: Union[str, List[int]], sampling_params: Optional[SamplingParams] = None) -> int:
+        if isinstance(prompt, str):
+            prompt = self._tokenizer().encode(prompt)
+        seq = Sequence(list(prompt), sampling_params)
+        self.scheduler.add(seq)
+        self._by_id[seq.seq_id] = seq
+        return seq.seq_id
+
+    def is_finished(self) -> bool:
+        return self.scheduler.is_finished()
+
+    def step(self) -> Tuple[List[Tuple[int, List[int]]], int]:
+        """One scheduling decision and one model step.  Returns the requests finished in it
+        as (id, completion token ids), and the token count of the step: positive for a step
+        of prompt tokens, minus the number of requests for a decode step (llm_engine.py:49-55)."""
+        t0 = perf_counter()
+        seqs, is_prefill = self.scheduler.schedule()
+        num_tokens = 0
+        if seqs:
+            entries, sampled = [], []
+            for seq in seqs:
+                start, n = seq.num_cached_tokens, seq.num_scheduled_tokens
+                last = start + n == seq.num_tokens
+                entries.append(StepEntry(seq.seq_id, seq.token_ids[start:start + n], start, [n - 1] if last else []))
+                if last:
+                    sampled.append(seq)
+            logits = self.runner.step(entries)
+            tokens = {}
+            if sampled:
+                ids = self.sampler.sample(
+                    logits, [s.temperature for s in sampled],
+                    [self.config.seed if s.seed is None else s.seed for s in sampled],
+                    [s.seq_id for s in sampled], [s.num_tokens for s in sampled])
+                tokens = {s.seq_id: t for s, t in zip(sampled, ids)}
+            elif self.model.device.type == "cuda":
+                torch.cuda.synchronize(self.model.device)
+            self.scheduler.postprocess(seqs, [tokens.get(s.seq_id, -1) for s in seqs])
+            num_tokens = sum(len(e.tokens) for e in entries) if is_prefill else -len(seqs)
+            dt = perf_counter() - t0
+            kind = "prefill" if is_prefill else "decode"
+            self.stats[f"{kind}_tokens"] += abs(num_tokens)
+            self.stats[f"{kind}_time"] += dt
+            self.stats["steps"] += 1
+        finished = self.scheduler.just_finished
+        self.scheduler.just_finished = []
+        outputs = [(s.seq_id, s.completion_token_ids) for s in finished]
+        return outputs, num_tokens
+
+    def generate(self, prompts: Seq[Union[str, List[int]]],
+                 sampling_params: Union[SamplingParams, Seq[SamplingParams], None] = None,
+                 use_tqdm: bool = True) -> List[dict]:
+        """llm_engine.py:60-90: returns, in the order of the prompts, {"text", "token_ids"}."""
+        if sampling_params is None:
+            sampling_params = SamplingParams()
+        if not isinstance(sampling_params, (list, tuple)):
+            sampling_params = [sampling_params] * len(prompts)
+        ids = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
+        done: Dict[int, List[int]] = {}
+        prefill_tps = decode_tps = 0.0
+        last_print = perf_counter()
+        while not self.is_finished():
+            t = perf_counter()
+            outputs, n = self.step()
+            dt = max(perf_counter() - t, 1e-9)
+            if n > 0:
+                prefill_tps = n / dt
+            elif n < 0:
+                decode_tps = -n / dt
+            for seq_id, toks in outputs:
+                done[seq_id] = toks
+            if use_tqdm and perf_counter() - last_print > 1.0:
+                last_print = perf_counter()
+                print(f"\rGenerating: {len(done)}/{len(ids)}  Prefill {int(prefill_tps)} tok/s  "
+                      f"Decode {int(decode_tps)} tok/s", end="", file=sys.stderr, flush=True)
+        if use_tqdm:
+            print(f"\rGenerating: {len(done)}/{len(ids)} done" + " " * 40, file=sys.stderr, flush=True)
+        self.model.kernels.check_faults()
+        results = []
+        for seq_id in ids:
+            toks = done[seq_id]
+            seq = self._by_id.pop(seq_id)
+            text = None
+            if self.tokenizer is not None:
+                text = self.tokenizer.decode(toks)
+            results.append({"text": text, "token_ids": toks, "finish_reason": seq.finish_reason})
+        return results
+
+    def exit(self):
+        pass

@@ -1,0 +1,172 @@
+"""Shared by the tests: tiny configurations, model folders, and the four ways of driving a
+request through the step function (whole; most of it then the last tokens one by one; in
+portions of changing size; mixed with other requests on few pages)."""
+from __future__ import annotations
+
+import os
+import random
+import tempfile
+from typing import Dict, List, Sequence
+
+import torch
+
+from nano_vllm_amd.config import Qwen3Config
+from nano_vllm_amd.engine.batch import StepEntry
+from nano_vllm_amd.engine.runner import ModelRunner
+from nano_vllm_amd.weights import write_random_model
+
+import plain_qwen3 as plain
+
+# Two BASELINE configurations and two more; together they differ in every size and option:
+# layers, width, heads and groups, head size, inner size, vocabulary, theta, eps, tying,
+# norm weights, page size.
+CONFIGS: Dict[str, dict] = {
+    "a": dict(cfg=Qwen3Config(vocab_size=256, hidden_size=64, num_hidden_layers=2, num_attention_heads=4,
+                              num_key_value_heads=2, head_dim=16, intermediate_size=128, rms_norm_eps=1e-6,
+                              rope_theta=10000.0, max_position_embeddings=128, tie_word_embeddings=True),
+              norm_std=0.0, page=4, seed=11),
+    "b": dict(cfg=Qwen3Config(vocab_size=384, hidden_size=96, num_hidden_layers=3, num_attention_heads=8,
+                              num_key_value_heads=2, head_dim=32, intermediate_size=160, rms_norm_eps=1e-5,
+                              rope_theta=1000000.0, max_position_embeddings=256, tie_word_embeddings=False),
+              norm_std=0.1, page=8, seed=12),
+    "c": dict(cfg=Qwen3Config(vocab_size=1000, hidden_size=120, num_hidden_layers=2, num_attention_heads=6,
+                              num_key_value_heads=3, head_dim=64, intermediate_size=200, rms_norm_eps=1e-6,
+                              rope_theta=500000.0, max_position_embeddings=1024, tie_word_embeddings=False),
+              norm_std=0.1, page=16, seed=13),
+    "d": dict(cfg=Qwen3Config(vocab_size=777, hidden_size=256, num_hidden_layers=2, num_attention_heads=8,
+                              num_key_value_heads=2, head_dim=128, intermediate_size=384, rms_norm_eps=1e-6,
+                              rope_theta=1000000.0, max_position_embeddings=2048, tie_word_embeddings=True),
+              norm_std=0.05, page=64, seed=14),
+}
+
+_folders: Dict[str, str] = {}
+_tmp = None
+
+
+def model_folder(name: str, dtype: str = "float32") -> str:
+    """A folder with config.json and model.safetensors of the named tiny configuration,
+    written once per test session into a temporary folder."""
+    global _tmp
+    key = f"{name}-{dtype}"
+    if key not in _folders:
+        if _tmp is None:
+            _tmp = tempfile.TemporaryDirectory(prefix="nva-models-")
+        c = CONFIGS[name]
+        path = os.path.join(_tmp.name, key)
+        write_random_model(path, c["cfg"], seed=c["seed"], norm_std=c["norm_std"], dtype=dtype)
+        _folders[key] = path
+    return _folders[key]
+
+
+def random_tokens(vocab: int, n: int, seed: int) -> List[int]:
+    rng = random.Random(seed)
+    return [rng.randrange(vocab) for _ in range(n)]
+
+
+def make_runner(folder: str, dtype: str, page: int, num_pages: int, device="cuda:0", kernels=None,
+                max_requests: int = 8) -> ModelRunner:
+    return ModelRunner.from_folder(folder, dtype=dtype, device=device, page_size=page, num_pages=num_pages,
+                                   max_requests=max_requests, kernels=kernels, quiet=True,
+                                   enable_prefix_caching=False)
+
+
+# ------------------------------------------------------------------------------ drivings
+def run_portions(runner: ModelRunner, rid, tokens: Sequence[int], portions: Sequence[int]) -> torch.Tensor:
+    """One request alone, cut into the given portions; logits of every position."""
+    assert sum(portions) == len(tokens)
+    runner.cache.admit(rid)
+    out, pos = [], 0
+    for n in portions:
+        runner.cache.reserve(rid, pos + n)
+        out.append(runner.step([StepEntry(rid, tokens[pos:pos + n], pos, list(range(n)))]).float().cpu())
+        pos += n
+    runner.cache.release(rid)
+    runner.cache.check()
+    return torch.cat(out)
+
+
+def whole(n: int) -> List[int]:
+    return [n]
+
+
+def last_one_by_one(n: int, last: int = 32) -> List[int]:
+    last = min(last, n - 1)
+    return [n - last] + [1] * last
+
+
+def changing_portions(n: int, seed: int) -> List[int]:
+    """Portions of changing size, down to two tokens (and ones at the end)."""
+    rng = random.Random(seed)
+    sizes, left = [], n
+    menu = [7, 2, 16, 3, 2, 33, 5, 2, 64, 9]
+    i = rng.randrange(len(menu))
+    while left > 0:
+        s = min(menu[i % len(menu)], left)
+        sizes.append(s)
+        left -= s
+        i += 1
+    return sizes
+
+
+def run_mixed(runner: ModelRunner, requests: Dict[str, List[int]], seed: int, max_live: int = 4):
+    """Up to max_live requests at a time: portions of some beside single decoded tokens of
+    others; a request that ends gives its pages back and a waiting one takes them.  Returns
+    {request: logits of every position}."""
+    rng = random.Random(seed)
+    waiting = list(requests)
+    live: Dict[str, int] = {}
+    got: Dict[str, List[torch.Tensor]] = {r: [] for r in requests}
+    decoding = set()
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            rid = waiting[0]
+            need = len(requests[rid])
+            pages_needed = (need + runner.page_size - 1) // runner.page_size
+            if runner.cache.pools[0].num_free - _reserved_pages(runner, live, requests) < pages_needed:
+                break
+            waiting.pop(0)
+            runner.cache.admit(rid)
+            live[rid] = 0
+        assert live, "the pool is too small for any request"
+        entries = []
+        for rid, pos in live.items():
+            left = len(requests[rid]) - pos
+            if rid in decoding or left <= 32:
+                decoding.add(rid)
+                n = 1
+            else:
+                n = min(left - 32, rng.choice([2, 3, 5, 8, 13, 21, 40]))
+            runner.cache.reserve(rid, pos + n)
+            entries.append(StepEntry(rid, requests[rid][pos:pos + n], pos, list(range(n))))
+        rng.shuffle(entries)
+        logits = runner.step(entries).float().cpu()
+        row = 0
+        for e in entries:
+            n = len(e.tokens)
+            got[e.request].append(logits[row:row + n])
+            row += n
+            live[e.request] += n
+            if live[e.request] == len(requests[e.request]):
+                runner.cache.release(e.request)
+                del live[e.request]
+                decoding.discard(e.request)
+        runner.cache.check()
+    return {r: torch.cat(v) for r, v in got.items()}
+
+
+def _reserved_pages(runner, live, requests) -> int:
+    """Pages that live requests will still take before they end."""
+    total = 0
+    for rid, pos in live.items():
+        full = (len(requests[rid]) + runner.page_size - 1) // runner.page_size
+        total += full - len(runner.cache.table(rid, 0))
+    return total
+
+
+def plain_logits(folder: str, tokens: Sequence[int], rounding=None) -> torch.Tensor:
+    cfg, w = plain.read_folder(folder)
+    return plain.logits(w, cfg, list(tokens), rounding)
+
+
+def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
+    return float((got.double() - want.double()).abs().max() / want.double().abs().max())
