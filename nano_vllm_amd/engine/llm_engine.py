@@ -48,6 +48,7 @@ class LLMEngine:
         self.sampler = Sampler(self.model.kernels, self.model.device)
         self.stats = {"prefill_tokens": 0, "prefill_time": 0.0, "decode_tokens": 0, "decode_time": 0.0, "steps": 0}
         self._by_id: Dict[int, Sequence] = {}
+        self._next_id = 0
 
     # ------------------------------------------------------------------ set-up helpers
     def _pages_from_free_memory(self) -> int:
@@ -100,7 +101,8 @@ class LLMEngine:
     def add_request(self, prompt: Union[str, List[int]], sampling_params: Optional[SamplingParams] = None) -> int:
         if isinstance(prompt, str):
             prompt = self._tokenizer().encode(prompt)
-        seq = Sequence(list(prompt), sampling_params)
+        seq = Sequence(list(prompt), sampling_params, seq_id=self._next_id)
+        self._next_id += 1
         self.scheduler.add(seq)
         self._by_id[seq.seq_id] = seq
         return seq.seq_id

@@ -21,11 +21,14 @@ class SequenceStatus(Enum):
 class Sequence:
     _ids = count()
 
-    def __init__(self, token_ids: List[int], sampling_params: Optional[SamplingParams] = None):
+    def __init__(self, token_ids: List[int], sampling_params: Optional[SamplingParams] = None,
+                 seq_id: Optional[int] = None):
         if not token_ids:
             raise ValueError("a request needs at least one prompt token")
         sp = sampling_params or SamplingParams()
-        self.seq_id = next(Sequence._ids)
+        # The reference numbers requests with one counter per process (sequence.py:16,19); an
+        # engine numbers its own from 0, so that equal runs draw equal sampling noise.
+        self.seq_id = next(Sequence._ids) if seq_id is None else seq_id
         self.status = SequenceStatus.WAITING
         self.token_ids = list(token_ids)
         self.num_prompt_tokens = len(token_ids)

@@ -1,0 +1,218 @@
+"""The cache manager on the host: no page is lost, held twice or freed twice, under random
+orders of requests; windows give pages back; freed pages are used again in order; prefix
+hashes; state slots."""
+import random
+from types import SimpleNamespace
+
+import pytest
+
+from nano_vllm_amd.cache import (CacheGroup, CacheManager, OutOfPages, PageError, PagePool, SlotPool, chain_hash,
+                                 plan_groups)
+from nano_vllm_amd.parts.spec import FixedState, PagedKV
+
+
+def _manager(pages=8, page=4, groups=(None,), slots=0, prefix=True):
+    gs = [CacheGroup(w, (i,)) for i, w in enumerate(groups)]
+    return CacheManager(gs, page, pages, num_state_slots=slots, has_state=slots > 0, enable_prefix_caching=prefix)
+
+
+def test_plan_groups_by_need():
+    needs = [PagedKV(2, 16), PagedKV(2, 16, window=8), None, PagedKV(4, 32), FixedState({"s": ((3,), "float32")}),
+             PagedKV(2, 16, window=8), PagedKV(2, 16, window=32)]
+    groups, state = plan_groups(needs)
+    assert [(g.window, g.runs) for g in groups] == [(None, (0, 3)), (8, (1, 5)), (32, (6,))]
+    assert state == [4]
+
+
+def test_pages_are_taken_and_given_back():
+    m = _manager(pages=4, page=4)
+    m.admit("a")
+    m.reserve("a", 5)
+    assert m.table("a", 0) == [0, 1] and m.pools[0].num_free == 2
+    m.reserve("a", 8)                                  # the same two pages suffice
+    assert m.table("a", 0) == [0, 1]
+    m.reserve("a", 9)
+    assert m.table("a", 0) == [0, 1, 2]
+    m.check()
+    m.release("a")
+    assert m.pools[0].num_free == 4
+    m.check()
+
+
+def test_freed_pages_are_used_again_oldest_first_and_tails_before_heads():
+    m = _manager(pages=4, page=2)
+    m.admit("a"); m.reserve("a", 6)                    # pages 0 1 2
+    m.release("a")                                     # freed in the order 2 1 0, behind the never-used 3
+    m.admit("b"); m.reserve("b", 8)
+    assert m.table("b", 0) == [3, 2, 1, 0]             # block_manager.py:43-56,94-101
+
+
+def test_out_of_pages_leaves_the_request_as_it_was():
+    m = _manager(pages=3, page=4)
+    m.admit("a"); m.reserve("a", 8)
+    m.admit("b")
+    assert not m.can_reserve("b", 8)
+    with pytest.raises(OutOfPages):
+        m.reserve("b", 8)
+    assert m.table("b", 0) == [] and m.pools[0].num_free == 1
+    m.check()
+    m.reserve("b", 4)
+    m.check()
+
+
+def test_freeing_twice_is_an_error():
+    pool = PagePool(2, 4)
+    p = pool.take()
+    pool.give_back(p)
+    with pytest.raises(PageError):
+        pool.give_back(p)
+    m = _manager()
+    m.admit("a")
+    m.release("a")
+    with pytest.raises(KeyError):
+        m.release("a")
+    m.admit("b")
+    with pytest.raises(PageError):
+        m.admit("b")
+
+
+def test_window_gives_passed_pages_back():
+    m = _manager(pages=4, page=4, groups=(None, 6))
+    m.admit("a")
+    pos = 0
+    for n in (5, 3, 4, 1, 1, 1, 1):                     # portions, then single tokens
+        m.reserve("a", pos + n, first_query=pos)
+        pos += n
+        full, win = m.table("a", 0), m.table("a", 1)
+        assert all(p >= 0 for p in full) and len(full) == (pos + 3) // 4
+        first_needed = max(0, (pos - n) - 6 + 1) // 4   # oldest key the step's first query reads
+        assert all(p == -1 for p in win[:first_needed]) and all(p >= 0 for p in win[first_needed:])
+        m.check()
+    assert m.table("a", 1)[:2] == [-1, -1]
+    assert m.pools[1].num_free == 4 - 2
+    m.release("a")
+    m.check()
+    assert m.pools[0].num_free == 4 and m.pools[1].num_free == 4
+
+
+def test_window_group_lets_a_long_request_live_on_few_pages():
+    m = _manager(pages=3, page=4, groups=(8,))
+    m.admit("a")
+    for pos in range(0, 100):
+        m.reserve("a", pos + 1, first_query=pos)        # never more than 3 pages held
+        m.check()
+    assert sum(1 for p in m.table("a", 0) if p >= 0) <= 3
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_random_orders_never_lose_or_double_a_page(seed):
+    rng = random.Random(seed)
+    m = _manager(pages=24, page=4, groups=(None, 10), slots=6, prefix=False)
+    live = {}
+    for step in range(600):
+        op = rng.random()
+        if op < 0.25 and len(live) < 6:
+            rid = f"r{step}"
+            m.admit(rid)
+            live[rid] = 0
+        elif op < 0.85 and live:
+            rid = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 2, 3, 7, 12])
+            new_len = live[rid] + n
+            if m.can_reserve(rid, new_len, first_query=live[rid]):
+                m.reserve(rid, new_len, first_query=live[rid])
+                live[rid] = new_len
+            else:
+                with pytest.raises(OutOfPages):
+                    m.reserve(rid, new_len, first_query=live[rid])
+        elif live:
+            rid = rng.choice(list(live))
+            m.release(rid)
+            del live[rid]
+        m.check()
+        for rid, n in live.items():
+            assert len(m.table(rid, 0)) == (n + 3) // 4
+    for rid in list(live):
+        m.release(rid)
+    m.check()
+    assert all(pool.num_free == pool.num_pages for pool in m.pools) and m.slots.num_free == 6
+
+
+# ------------------------------------------------------------------------------ prefix hashes
+def test_chain_hash_depends_on_the_prefix():
+    a = chain_hash([1, 2, 3, 4])
+    assert a == chain_hash([1, 2, 3, 4]) and a != chain_hash([1, 2, 3, 5])
+    assert chain_hash([5, 6, 7, 8], a) != chain_hash([5, 6, 7, 8])
+
+
+def test_prefix_pages_are_found_and_shared_but_never_the_last():
+    m = _manager(pages=8, page=4)
+    toks = list(range(10, 22))                         # 12 tokens = 3 full pages
+    assert m.can_admit(toks) == 0
+    assert m.admit_with_prefix("a", toks) == 0
+    m.register_full_pages("a", toks, 12)
+    # an equal prompt: the first two pages are shared, the last one is computed again (block_manager.py:62)
+    assert m.can_admit(toks) == 2
+    assert m.admit_with_prefix("b", toks) == 8
+    assert m.table("b", 0)[:2] == m.table("a", 0)[:2] and m.table("b", 0)[2] != m.table("a", 0)[2]
+    assert m.pools[0].ref_count[m.table("a", 0)[0]] == 2
+    m.check()
+    # a prompt that differs inside the second page shares only the first
+    other = toks[:5] + [99] + toks[6:]
+    assert m.can_admit(other) == 1
+    m.release("a")
+    m.check()
+    assert m.pools[0].ref_count[m.table("b", 0)[0]] == 1
+    m.release("b")
+    m.check()
+    # freed pages stay findable until they are taken again (block_manager.py:43-51)
+    assert m.can_admit(toks + [1]) == 3
+    assert m.admit_with_prefix("c", toks + [1]) == 12
+    m.check()
+
+
+def test_a_hit_needs_equal_tokens_not_only_an_equal_hash():
+    m = _manager(pages=4, page=2)
+    m.admit_with_prefix("a", [1, 2, 3])
+    m.register_full_pages("a", [1, 2, 3], 3)
+    page = m.table("a", 0)[0]
+    m.pools[0].tokens_of[page] = (7, 7)                 # as after a hash collision
+    assert m.can_admit([1, 2, 3]) == 0
+
+
+def test_a_hit_on_a_free_page_still_takes_it():
+    m = _manager(pages=4, page=2)
+    toks = [1, 2, 3, 4, 5]
+    m.admit_with_prefix("a", toks)
+    m.register_full_pages("a", toks, 5)
+    m.release("a")                                      # free list: 3 (never used), then a's 2, 1, 0
+    m.admit("x"); m.reserve("x", 2)                     # takes page 3
+    assert m.can_admit(toks) == 2                       # both hashed pages are still there, free: 3 free pages suffice
+    m.admit("y"); m.reserve("y", 2)                     # takes a's unhashed tail page
+    assert m.can_admit(toks) == -1                      # 3 pages wanted, hits are free pages themselves: 2 free < 3
+    assert m.can_admit(toks[:4]) == 1                   # 2 pages wanted, 2 free (one of them the hit)
+    m.check()
+
+
+def test_prefix_caching_is_off_with_windows_or_state():
+    assert _manager(groups=(None, 8)).prefix_caching is False
+    assert _manager(slots=2).prefix_caching is False
+    assert _manager(prefix=False).prefix_caching is False
+    assert _manager().prefix_caching is True
+
+
+# ------------------------------------------------------------------------------ state slots
+def test_state_slots():
+    m = _manager(slots=2)
+    a, b = m.admit("a"), m.admit("b")
+    assert {a.state_slot, b.state_slot} == {0, 1}
+    with pytest.raises(OutOfPages):
+        m.admit("c")
+    m.release("a")
+    assert m.admit("c").state_slot == a.state_slot
+    m.check()
+    pool = SlotPool(1)
+    s = pool.take()
+    pool.give_back(s)
+    with pytest.raises(PageError):
+        pool.give_back(s)

@@ -1,0 +1,134 @@
+"""The engine's host logic (batching, block tables, slot mapping, scheduler, engine loop)
+on the CPU: the device operations are replaced by their plain torch versions
+(tests/torch_kernels.py), the model and everything above it is the product's.  Compared
+with the plain implementation in float32."""
+import pytest
+import torch
+
+import helpers as H
+import plain_qwen3 as plain
+from nano_vllm_amd import LLM, SamplingParams
+from nano_vllm_amd.cache import OutOfPages
+from nano_vllm_amd.engine.batch import StepEntry
+from torch_kernels import TorchKernels
+
+TOL = 2e-5
+
+
+def _runner(name, pages):
+    c = H.CONFIGS[name]
+    return H.make_runner(H.model_folder(name), "float32", c["page"], pages, device="cpu", kernels=TorchKernels())
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_every_cutting_gives_the_plain_logits(name):
+    c = H.CONFIGS[name]
+    n = 70
+    toks = H.random_tokens(c["cfg"].vocab_size, n, 1)
+    want = H.plain_logits(H.model_folder(name), toks)
+    r = _runner(name, 32)
+    for portions in (H.whole(n), H.last_one_by_one(n), H.changing_portions(n, 2)):
+        got = H.run_portions(r, "x", toks, portions)
+        assert H.rel_err(got, want) < TOL, portions
+
+
+def test_mixed_batches_on_few_pages():
+    c = H.CONFIGS["b"]
+    lens = {"r0": 60, "r1": 41, "r2": 77, "r3": 35, "r4": 52, "r5": 66}
+    reqs = {r: H.random_tokens(c["cfg"].vocab_size, n, i) for i, (r, n) in enumerate(lens.items())}
+    r = _runner("b", 26)                  # 208 tokens of cache for 331 tokens of requests: pages are used again
+    got = H.run_mixed(r, reqs, seed=3)
+    for rid, toks in reqs.items():
+        assert H.rel_err(got[rid], H.plain_logits(H.model_folder("b"), toks)) < TOL, rid
+    assert r.cache.pools[0].num_free == 26
+
+
+def test_step_refuses_what_the_cache_does_not_hold():
+    r = _runner("a", 4)
+    r.cache.admit("x")
+    r.cache.reserve("x", 3)
+    with pytest.raises(ValueError, match="not reserved"):
+        r.step([StepEntry("x", [1, 2, 3, 4], 0, [])])
+    with pytest.raises(ValueError, match="vocabulary"):
+        r.step([StepEntry("x", [1, 2, 999], 0, [])])
+    with pytest.raises(ValueError, match="twice"):
+        r.step([StepEntry("x", [1], 0, []), StepEntry("x", [2], 1, [])])
+    with pytest.raises(ValueError, match="wanted place"):
+        r.step([StepEntry("x", [1, 2], 0, [2])])
+    assert r.step([StepEntry("x", [1, 2], 0, [])]) is None
+    with pytest.raises(OutOfPages):
+        r.cache.reserve("x", 17)
+
+
+def test_logits_come_back_in_the_callers_order():
+    c = H.CONFIGS["a"]
+    r = _runner("a", 16)
+    t1, t2 = H.random_tokens(256, 9, 1), H.random_tokens(256, 6, 2)
+    w1, w2 = H.plain_logits(H.model_folder("a"), t1), H.plain_logits(H.model_folder("a"), t2)
+    for rid, n in (("p", 9), ("q", 6)):
+        r.cache.admit(rid)
+        r.cache.reserve(rid, n)
+    r.step([StepEntry("q", t2[:5], 0, [])])
+    # a portion first, a single token second: the step reorders, the answer does not
+    out = r.step([StepEntry("p", t1, 0, [8, 0, 3]), StepEntry("q", t2[5:], 5, [0])])
+    want = torch.stack([w1[8], w1[0], w1[3], w2[5]])
+    assert H.rel_err(out, want) < TOL
+
+
+def _llm(name, **kw):
+    c = H.CONFIGS[name]
+    opts = dict(kernels=TorchKernels(), device="cpu", dtype="float32", kvcache_block_size=c["page"],
+                num_kvcache_blocks=64, max_num_batched_tokens=16, max_num_seqs=4)
+    opts.update(kw)
+    return LLM(H.model_folder(name), **opts)
+
+
+def _prompts(name, lens):
+    return [H.random_tokens(H.CONFIGS[name]["cfg"].vocab_size, n, 100 + n) for n in lens]
+
+
+def test_greedy_generation_is_the_plain_argmax_chain():
+    prompts = _prompts("b", (3, 9, 24, 40))
+    outs = _llm("b").generate(prompts, SamplingParams(temperature=0.0, max_tokens=8), use_tqdm=False)
+    cfg, w = plain.read_folder(H.model_folder("b"))
+    for p, o in zip(prompts, outs):
+        assert o["token_ids"] == plain.greedy_generate(w, cfg, p, 8)
+        assert o["finish_reason"] == "max_tokens" and o["text"] is None
+
+
+def test_schedules_prefix_cache_and_page_shortage_do_not_change_the_tokens():
+    prompts = _prompts("b", (3, 9, 24, 40))
+    shared = prompts[3][:32]
+    prompts += [shared + [5, 6, 7], shared + [9]]            # two requests with four pages in common
+    sp = [SamplingParams(temperature=0.0, max_tokens=10), SamplingParams(temperature=0.7, max_tokens=10)] * 3
+    base = _llm("b", enable_prefix_caching=False).generate(prompts, sp, use_tqdm=False)
+    for kw in (dict(schedule="mixed"), dict(enable_prefix_caching=True), dict(num_kvcache_blocks=14),
+               dict(num_kvcache_blocks=14, schedule="mixed"), dict(max_num_batched_tokens=5, max_num_seqs=2)):
+        llm = _llm("b", **kw)
+        outs = llm.generate(prompts, sp, use_tqdm=False)
+        assert [o["token_ids"] for o in outs] == [o["token_ids"] for o in base], kw
+        llm.runner.cache.check()
+        assert llm.runner.cache.pools[0].num_free == llm.config.num_kvcache_blocks
+        if kw.get("num_kvcache_blocks") == 14:
+            assert llm.scheduler.num_preemptions > 0
+
+
+def test_temperature_sampling_is_the_plain_draw_and_is_reproducible():
+    prompts = _prompts("a", (5, 11))
+    sp = SamplingParams(temperature=0.7, max_tokens=5, seed=42)
+    llm = _llm("a")
+    outs = llm.generate(prompts, sp, use_tqdm=False)
+    cfg, w = plain.read_folder(H.model_folder("a"))
+    # by hand: the same seed, request number and position give the same noise
+    for k, (p, o) in enumerate(zip(prompts, outs)):
+        toks = list(p)
+        for _ in range(5):
+            l = plain.logits(w, cfg, toks)[-1]
+            toks.append(plain.sample(l, 0.7, seed=42, request=k, position=len(toks)))
+        assert o["token_ids"] == toks[len(p):]
+    assert [o["token_ids"] for o in _llm("a").generate(prompts, sp, use_tqdm=False)] == [o["token_ids"] for o in outs]
+
+
+def test_unknown_option_is_an_error():
+    with pytest.raises(TypeError, match="unknown engine options"):
+        _llm("a", max_batch=3)
