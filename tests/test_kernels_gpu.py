@@ -1,0 +1,328 @@
+"""Each HIP kernel alone against its plain torch version (tests/torch_kernels.py), in
+float32 and bfloat16, at sizes other than the engine's tiny models: widths and vocabularies
+that are no power of two, head sizes in steps of 16, odd numbers of heads and groups, page
+sizes from 4 to 256, rows that are not aligned for vector access."""
+import math
+import random
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+import plain_qwen3 as plain
+from torch_kernels import TorchKernels
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def hip():
+    from nano_vllm_amd.kernels import HipKernels
+    return {dt: HipKernels(DEV, dt, quiet=True) for dt in DTYPES}
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return TorchKernels(DEV)
+
+
+def _close(got, want, dtype, what=""):
+    got, want = got.float(), want.float()
+    scale = float(want.abs().max()) or 1.0
+    tol = 2e-6 if dtype == torch.float32 else 2.0 ** -7          # two units in the last place of bfloat16
+    err = float((got - want).abs().max()) / scale
+    assert err <= tol, f"{what}: error {err:.3e} of the largest value exceeds {tol:.1e}"
+
+
+def _rand(shape, dtype, seed, scale=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (scale * torch.randn(shape, generator=g)).to(dtype).to(DEV)
+
+
+# ------------------------------------------------------------------------------ rows
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,width,n", [(50, 100, 7), (1000, 4096, 33), (17, 6, 5), (300, 1001, 64)])
+def test_embedding(hip, ref, dtype, rows, width, n):
+    table = _rand((rows, width), dtype, 1)
+    ids = torch.randint(0, rows, (n,), dtype=torch.int32, device=DEV)
+    assert torch.equal(hip[dtype].embedding(table, ids), ref.embedding(table, ids))
+    # a strided view of a wider tensor (rows not aligned for vector access)
+    wide = _rand((rows, width + 3), dtype, 2)
+    assert torch.equal(hip[dtype].embedding(wide[:, 1:width + 1], ids), wide[:, 1:width + 1][ids.long()])
+
+
+def test_embedding_flags_an_id_outside_the_table(hip):
+    from nano_vllm_amd.kernels import KernelError
+    k = hip[torch.float32]
+    table = _rand((10, 8), torch.float32, 1)
+    out = k.embedding(table, torch.tensor([3, 10, -1], dtype=torch.int32, device=DEV))
+    assert torch.equal(out[0], table[3]) and float(out[1:].abs().max()) == 0.0
+    with pytest.raises(KernelError, match="vocabulary"):
+        k.check_faults()
+    k.check_faults()                                              # the flag is cleared
+
+
+# ------------------------------------------------------------------------------ norms
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,width", [(1, 7), (5, 96), (33, 120), (3, 4096), (2, 5120), (4, 1001)])
+@pytest.mark.parametrize("weight32", [False, True])
+def test_rms_norm_and_fused_add(hip, ref, dtype, rows, width, weight32):
+    x, r = _rand((rows, width), dtype, 3, 2.0), _rand((rows, width), dtype, 4, 3.0)
+    w = (1 + 0.1 * torch.randn(width)).to(torch.float32 if weight32 else dtype).to(DEV)
+    _close(hip[dtype].rms_norm(x, w, 1e-5), ref.rms_norm(x, w, 1e-5), dtype, "rms_norm")
+    r1, r2 = r.clone(), r.clone()
+    y1, _ = hip[dtype].add_rms_norm(x, r1, w, 1e-6)
+    y2, _ = ref.add_rms_norm(x, r2, w, 1e-6)
+    _close(y1, y2, dtype, "add_rms_norm")
+    _close(r1, r2, dtype, "residual")
+    # in place on the input, as the block calls it
+    x2 = x.clone()
+    y3, _ = hip[dtype].add_rms_norm(x2, r.clone(), w, 1e-6, out=x2)
+    assert torch.equal(y3, y1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_rms_norm_on_strided_rows(hip, ref, dtype):
+    big = _rand((6, 300), dtype, 5)
+    x = big[:, 3:203]                                              # unaligned start, stride 300
+    w = _rand((200,), dtype, 6)
+    _close(hip[dtype].rms_norm(x, w, 1e-6), ref.rms_norm(x, w, 1e-6), dtype)
+
+
+# ------------------------------------------------------------------------------ feed-forward
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,inner", [(1, 5), (7, 160), (3, 12288), (40, 1000)])
+def test_silu_mul(hip, ref, dtype, rows, inner):
+    x = _rand((rows, 2 * inner), dtype, 7, 2.0)
+    _close(hip[dtype].silu_mul(x), ref.silu_mul(x), dtype)
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 7, 5), (3, 130, 67), (65, 64, 128), (200, 300, 1000), (2, 1001, 96), (64, 96, 4096)])
+def test_linear_float32(hip, ref, m, n, k):
+    x, w = _rand((m, k), torch.float32, 8), _rand((n, k), torch.float32, 9)
+    want = x.double() @ w.double().T
+    # a float sum of k terms: each output may be off by about sqrt(k) roundings of its |terms|
+    bound = (x.double().abs() @ w.double().abs().T) * (math.sqrt(k) * 2.0 ** -23) + 1e-30
+    got = hip[torch.float32].linear(x, w).double()
+    assert bool(((got - want).abs() <= bound).all()), float(((got - want).abs() / bound).max())
+    b = _rand((n,), torch.float32, 10)
+    got = hip[torch.float32].linear(x, w, b).double()
+    assert bool(((got - want - b.double()).abs() <= bound + b.double().abs() * 2.0 ** -23).all())
+
+
+def test_linear_float32_does_not_depend_on_the_rows_beside_it(hip):
+    x, w = _rand((70, 333), torch.float32, 11), _rand((129, 333), torch.float32, 12)
+    k = hip[torch.float32]
+    whole = k.linear(x, w)
+    assert torch.equal(k.linear(x[17:18], w), whole[17:18])         # bit for bit: the order of the sum is fixed
+    assert torch.equal(k.linear(x[:3], w), whole[:3])
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1001, 96), (5, 384, 120), (70, 777, 256), (3, 64, 4096)])
+def test_linear_bfloat16_with_float_result(hip, m, n, k):
+    x, w = _rand((m, k), torch.bfloat16, 13), _rand((n, k), torch.bfloat16, 14)
+    got = hip[torch.bfloat16].linear(x, w, out_float32=True)
+    assert got.dtype == torch.float32
+    bound = (x.double().abs() @ w.double().abs().T) * (math.sqrt(k) * 2.0 ** -23) + 1e-30
+    assert bool(((got.double() - x.double() @ w.double().T).abs() <= bound).all())
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 130, 67), (8, 96, 200), (300, 257, 120)])
+def test_linear_bfloat16(hip, ref, m, n, k):
+    x, w = _rand((m, k), torch.bfloat16, 15), _rand((n, k), torch.bfloat16, 16)
+    _close(hip[torch.bfloat16].linear(x, w), ref.linear(x, w), torch.bfloat16)
+
+
+# ------------------------------------------------------------------------------ rotation and cache write
+def _inv_freq(D, theta):
+    return (1.0 / (theta ** (torch.arange(0, D, 2, dtype=torch.float) / D))).to(DEV)
+
+
+@pytest.mark.parametrize("D,theta,P", [(16, 1e4, 128), (48, 5e5, 300), (128, 1e6, 4096)])
+def test_rotary_table(hip, D, theta, P):
+    inv = _inv_freq(D, theta)
+    t = hip[torch.float32].rotary_table(inv, P)
+    ang = plain.rope_angles(D, torch.arange(P), theta)                # the reference's float32 angles, on the CPU
+    assert float((t[:, : D // 2].cpu() - ang.cos()).abs().max()) < 2e-6
+    assert float((t[:, D // 2:].cpu() - ang.sin()).abs().max()) < 2e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,D,page,norm", [(4, 2, 16, 4, True), (5, 5, 48, 16, True), (6, 2, 64, 8, False),
+                                                 (7, 1, 80, 64, True), (8, 2, 128, 256, True), (3, 3, 256, 32, True)])
+def test_qk_norm_rope_store(hip, ref, dtype, hq, hkv, D, page, norm):
+    T = 37
+    pages = (T + page - 1) // page + 2
+    k = hip[dtype]
+    qkv = _rand((T, (hq + 2 * hkv) * D), dtype, 17)
+    qw = _rand((D,), dtype, 18) + 1 if norm else None
+    kw = _rand((D,), dtype, 19) + 1 if norm else None
+    table = ref.rotary_table(_inv_freq(D, 1e4), 500)
+    positions = torch.randint(0, 500, (T,), dtype=torch.int32, device=DEV)
+    slots = torch.randperm(pages * page)[:T].to(torch.int32).to(DEV)
+    slots[5] = -1                                                   # this token is not stored
+    caches = [[torch.zeros((pages, hkv, page, D), dtype=dtype, device=DEV),
+               torch.zeros((pages, hkv, D, page), dtype=dtype, device=DEV)] for _ in range(2)]
+    a, b = qkv.clone(), qkv.clone()
+    qa = k.qk_norm_rope_store(a, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[0])
+    qb = ref.qk_norm_rope_store(b, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[1])
+    _close(qa, qb, dtype, "q")
+    _close(a, b, dtype, "k in place")
+    _close(caches[0][0], caches[1][0], dtype, "k cache")
+    assert torch.equal(caches[0][1], caches[1][1])                  # values are copied as they are
+    assert float(caches[0][0].abs().sum()) > 0
+    # without norm weights and table the kernel only stores
+    c = qkv.clone()
+    k.qk_norm_rope_store(c, hq, hkv, D, None, None, 1e-6, None, None, slots, *caches[0])
+    assert torch.equal(c, qkv)
+
+
+def test_qk_refusals(hip):
+    from nano_vllm_amd.kernels import KernelError
+    k = hip[torch.float32]
+    with pytest.raises(KernelError, match="width"):
+        k.qk_norm_rope_store(torch.zeros((2, 100), device=DEV), 2, 1, 16, None, None, 1e-6, None, None, None, None, None)
+    with pytest.raises(KernelError, match="head_dim"):
+        k.qk_norm_rope_store(torch.zeros((2, 4 * 1024), device=DEV), 2, 1, 1024, None, None, 1e-6, None, None, None, None, None)
+
+
+# ------------------------------------------------------------------------------ attention
+def _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed, boost=None):
+    """A batch of requests with kv lengths `lens`, the last q_lens of which are this step's
+    queries; keys and values scattered over shuffled pages."""
+    rng = random.Random(seed)
+    S = len(lens)
+    pages_per = [(n + page - 1) // page for n in lens]
+    total = sum(pages_per) + 3
+    order = list(range(total))
+    rng.shuffle(order)
+    kc = torch.zeros((total, hkv, page, D), dtype=dtype, device=DEV)
+    vc = torch.zeros((total, hkv, D, page), dtype=dtype, device=DEV)
+    kc.normal_(0, 1.0)                                              # what unused slots hold must not matter
+    vc.normal_(0, 1.0)
+    width = max(pages_per)
+    tables = torch.full((S, width), -1, dtype=torch.int32)
+    ks, vs, qs, token_seq, positions = [], [], [], [], []
+    for s, n in enumerate(lens):
+        mine = [order.pop() for _ in range(pages_per[s])]
+        tables[s, : len(mine)] = torch.tensor(mine, dtype=torch.int32)
+        k = _rand((n, hkv, D), dtype, seed * 100 + s)
+        v = _rand((n, hkv, D), dtype, seed * 100 + 50 + s)
+        q = _rand((n, hq, D), dtype, seed * 100 + 70 + s)
+        if boost is not None:                                       # one far key that every late query prefers
+            k[boost] = 0
+            k[boost, :, 0] = 8.0                                    # score 64; every other key: 8 * N(0, 1)
+            q[:] = 0
+            q[:, :, 0] = 8.0
+        for j in range(n):
+            kc[mine[j // page], :, j % page, :] = k[j]
+            vc[mine[j // page], :, :, j % page] = v[j]
+        ks.append(k); vs.append(v); qs.append(q)
+        token_seq += [s] * q_lens[s]
+        positions += list(range(n - q_lens[s], n))
+    q = torch.cat([qs[s][lens[s] - q_lens[s]:] for s in range(S)]).reshape(sum(q_lens), hq * D).contiguous()
+    batch = SimpleNamespace(
+        num_seqs=S, num_tokens=sum(q_lens), token_seq=torch.tensor(token_seq, dtype=torch.int32, device=DEV),
+        positions=torch.tensor(positions, dtype=torch.int32, device=DEV), max_kv_len=max(lens), max_q_len=max(q_lens),
+        kv_lens=torch.tensor(lens, dtype=torch.int32, device=DEV),
+        cu_seqlens_q=torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=DEV),
+        num_decode=sum(1 for n in q_lens if n == 1), q_lens=list(q_lens),
+        groups=[SimpleNamespace(block_tables=tables.to(DEV), slot_mapping=None)])
+    return q, kc, vc, batch, (qs, ks, vs)
+
+
+def _plain_attention(qs, ks, vs, lens, q_lens, scale, window=None):
+    out = []
+    for q, k, v, n, nq in zip(qs, ks, vs, lens, q_lens):
+        o = plain.causal_attention(q.float().cpu(), k.float().cpu(), v.float().cpu(), scale, window)
+        out.append(o[n - nq:].reshape(nq, -1))
+    return torch.cat(out)
+
+
+ATT_CASES = [
+    # hq, hkv, D, page, kv lens, q lens, window
+    (4, 2, 16, 4, [5, 11, 17], [5, 11, 17], None),                 # whole prompts
+    (8, 2, 32, 8, [40, 9, 24, 3], [1, 1, 16, 3], None),            # decode beside portions
+    (6, 3, 48, 16, [100, 33], [1, 20], None),
+    (5, 5, 80, 64, [130, 64, 65], [2, 64, 1], None),               # page edges
+    (8, 2, 128, 256, [700, 300, 257], [1, 1, 1], None),            # long decode
+    (7, 1, 64, 32, [90, 31], [45, 1], None),                       # seven heads on one kv head
+    (4, 2, 128, 16, [200, 50], [30, 1], 24),                       # window
+    (2, 1, 256, 8, [33], [33], 5),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,D,page,lens,q_lens,window", ATT_CASES)
+def test_paged_attention(hip, ref, dtype, hq, hkv, D, page, lens, q_lens, window):
+    q, kc, vc, batch, parts = _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed=3)
+    scale = D ** -0.5
+    got = hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window)
+    want = _plain_attention(*parts, lens, q_lens, scale, window).to(DEV)
+    _close(got, want.to(dtype), dtype, "against the plain whole-sequence attention")
+    twin = ref.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window)
+    _close(got, twin, dtype, "against the plain paged attention")
+    hip[dtype].check_faults()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_reads_a_far_key_among_hundreds(hip, dtype):
+    # key 3 scores far above all others for every query: the output must be its value
+    hq, hkv, D, page, lens, q_lens = 4, 2, 64, 16, [600], [40]
+    q, kc, vc, batch, (qs, ks, vs) = _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed=5, boost=3)
+    got = hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, 1.0, None).float()
+    want = vs[0][3].float().repeat_interleave(hq // hkv, 0).reshape(1, hq * D).expand(40, -1)
+    assert float((got - want).abs().max()) < 0.05
+    # with a window that ends after it, the far key is gone
+    got_w = hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, 1.0, 100).float()
+    assert float((got_w - want).abs().max()) > 0.5
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_window_edge(hip, dtype):
+    # exactly `window` keys are seen: the key at p - window is out, the one at p - window + 1 is in
+    hq, hkv, D, page, W = 2, 1, 32, 8, 16
+    for boost, inside in ((83, False), (84, True)):                 # the query stands at position 99
+        q, kc, vc, batch, (qs, ks, vs) = _paged_case(dtype, hq, hkv, D, page, [100], [1], seed=7, boost=boost)
+        got = hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, 1.0, W).float()
+        want = vs[0][boost].float().repeat_interleave(hq, 0).reshape(1, hq * D)
+        assert (float((got - want).abs().max()) < 0.05) == inside
+
+
+def test_attention_flags_a_missing_page(hip):
+    from nano_vllm_amd.kernels import KernelError
+    q, kc, vc, batch, _ = _paged_case(torch.float32, 2, 1, 16, 4, [10], [1], seed=1)
+    batch.groups[0].block_tables[0, 1] = -1
+    hip[torch.float32].paged_attention(q, 2, 1, 16, kc, vc, batch, 0, 1.0, None)
+    with pytest.raises(KernelError, match="page"):
+        hip[torch.float32].check_faults()
+
+
+# ------------------------------------------------------------------------------ sampling
+def test_sampling_matches_the_plain_draw(hip):
+    from nano_vllm_amd.sampling.sampler import noise_key
+    k = hip[torch.float32]
+    V, R = 1001, 6
+    logits = _rand((R, V), torch.float32, 20, 3.0)
+    logits[0, 17] = logits[0, 900] = 50.0                           # a tie: the lowest index wins
+    temps = torch.tensor([0.0, 0.0, 0.7, 1.0, 0.3, 1.5], device=DEV)
+    keys = torch.tensor([noise_key(9, r, 100 + r) for r in range(R)], dtype=torch.int64, device=DEV)
+    got = k.sample(logits, temps, keys).tolist()
+    want = [plain.sample(logits[r].cpu(), float(temps[r]), seed=9, request=r, position=100 + r) for r in range(R)]
+    assert got == want and got[0] == 17
+
+
+def test_sampling_frequencies_follow_the_softmax(hip):
+    from nano_vllm_amd.sampling.sampler import noise_key
+    l = torch.tensor([1.0, 0.0, -1.0, 0.5, -2.0, 0.2, -0.3])
+    n, T = 20000, 0.8
+    logits = l.to(DEV).repeat(n, 1)
+    keys = torch.tensor([noise_key(1, 0, i) for i in range(n)], dtype=torch.int64, device=DEV)
+    got = hip[torch.float32].sample(logits, torch.full((n,), T, device=DEV), keys)
+    counts = torch.bincount(got.long().cpu(), minlength=7).double()
+    p = torch.softmax(l.double() / T, 0)
+    chi2 = float(((counts - n * p) ** 2 / (n * p)).sum())
+    assert chi2 < 22.5                                              # 6 degrees of freedom, 0.1 % point

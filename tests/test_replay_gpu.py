@@ -1,0 +1,149 @@
+"""The engine on the GPU against the plain implementation, in float32 and bfloat16: each
+request alone and whole; most of it in one step and the last 32 tokens one by one; in
+portions of changing size, down to two tokens; mixed, up to four live requests on so few
+pages that they are used again; long decoding; the first tokens; and the same through
+bin/trace_run as a user calls it."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+# float32: summation order only.  bfloat16: both sides round at the same places (the plain
+# implementation emulates them), but sum in different orders, so single roundings of about
+# 2^-9 flip and travel through the layers; 2e-2 of the largest logit bounds what a few such
+# flips per layer give and is far below the effect of any indexing fault.
+TOL = {"float32": 2e-5, "bfloat16": 2e-2}
+ROUNDING = {"float32": None, "bfloat16": "bfloat16"}
+
+
+@pytest.fixture(scope="module")
+def runners():
+    made = {}
+
+    def get(name, dtype, pages):
+        key = (name, dtype, pages)
+        if key not in made:
+            made[key] = H.make_runner(H.model_folder(name, dtype), dtype, H.CONFIGS[name]["page"], pages)
+        return made[key]
+    return get
+
+
+def _length(name):
+    return min(H.CONFIGS[name]["cfg"].max_position_embeddings - 2, 250)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+@pytest.mark.parametrize("driving", ["whole", "last32", "portions"])
+def test_one_request(runners, name, dtype, driving):
+    n = _length(name)
+    toks = H.random_tokens(H.CONFIGS[name]["cfg"].vocab_size, n, 21)
+    want = H.plain_logits(H.model_folder(name, dtype), toks, ROUNDING[dtype])
+    portions = {"whole": H.whole(n), "last32": H.last_one_by_one(n), "portions": H.changing_portions(n, 5)}[driving]
+    r = runners(name, dtype, 80)
+    got = H.run_portions(r, "x", toks, portions)
+    assert H.rel_err(got, want) < TOL[dtype]
+    if dtype == "float32":
+        assert torch.equal(got.argmax(-1), want.argmax(-1))
+    r.kernels.check_faults()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["b", "c", "d"])
+def test_mixed_requests_on_few_pages(runners, name, dtype):
+    c = H.CONFIGS[name]
+    top = _length(name)
+    lens = [top, top // 2 + 3, top - 17, 40, top // 3, top - 40, 65]
+    reqs = {f"r{i}": H.random_tokens(c["cfg"].vocab_size, n, 30 + i) for i, n in enumerate(lens)}
+    need = sorted(((n + c["page"] - 1) // c["page"] for n in lens), reverse=True)
+    pages = sum(need[:3]) + 1                      # room for about three of the seven at a time
+    r = runners(name, dtype, pages)
+    got = H.run_mixed(r, reqs, seed=4)
+    for rid, toks in reqs.items():
+        want = H.plain_logits(H.model_folder(name, dtype), toks, ROUNDING[dtype])
+        assert H.rel_err(got[rid], want) < TOL[dtype], rid
+    assert r.cache.pools[0].num_free == pages
+    r.kernels.check_faults()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(runners, dtype):
+    name = "c"
+    n = 600
+    toks = H.random_tokens(H.CONFIGS[name]["cfg"].vocab_size, n, 41)
+    want = H.plain_logits(H.model_folder(name, dtype), toks, ROUNDING[dtype])
+    r = runners(name, dtype, 80)
+    got = H.run_portions(r, "x", toks, [1] * n)     # every token decoded, from the very first
+    assert H.rel_err(got[:8], want[:8]) < TOL[dtype]
+    assert H.rel_err(got, want) < TOL[dtype]
+
+
+def test_logits_do_not_depend_on_pages_or_batch_mates(runners):
+    """float32: the same request alone, beside others, and on other pages gives the same
+    logits to the last bit (every sum runs in an order that the batch does not change)."""
+    name = "b"
+    c = H.CONFIGS[name]
+    toks = H.random_tokens(c["cfg"].vocab_size, 90, 51)
+    r = runners(name, "float32", 80)
+    alone = H.run_portions(r, "x", toks, H.changing_portions(90, 1))
+    others = {f"o{i}": H.random_tokens(c["cfg"].vocab_size, 50 + 9 * i, 60 + i) for i in range(3)}
+    mixed = H.run_mixed(r, {"o0": others["o0"], "x": toks, "o1": others["o1"], "o2": others["o2"]}, seed=8)
+    assert torch.equal(mixed["x"], alone)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_as_a_user_calls_it(tmp_path, dtype):
+    """bin/trace_run in a process of its own: portions, single tokens, four live requests,
+    a pool so small that pages are used again."""
+    name = "b"
+    c = H.CONFIGS[name]
+    folder = H.model_folder(name, dtype)
+    lens = {"a": 100, "b": 70, "c": 130, "d": 64, "e": 90}
+    reqs = {k: H.random_tokens(c["cfg"].vocab_size, n, 70 + i) for i, (k, n) in enumerate(lens.items())}
+    # steps: a and b start; c joins; a ends, d takes its pages; ...
+    plan = [
+        [("a", 60), ("b", 2)], [("a", 38), ("b", 33), ("c", 64)], [("a", 1), ("b", 1), ("c", 2)],
+        [("a", 1), ("b", 34), ("c", 64)], "end:a", [("d", 63), ("b", 0), ("c", 0)], [("d", 1), ("e", 7)],
+        "end:b", [("e", 83)], "end:c,d,e",
+    ]
+    pos = {k: 0 for k in reqs}
+    lines, wants, step = [], {}, 0
+    pending_end = []
+    for item in plan:
+        if isinstance(item, str):
+            lines[-1]["end"] = item[4:].split(",")
+            continue
+        entries = []
+        for rid, n in item:
+            if n == 0:
+                continue
+            want = list(range(n)) if n <= 4 else [0, n // 2, n - 1]
+            entries.append({"id": rid, "tokens": reqs[rid][pos[rid]:pos[rid] + n], "want": want})
+            for w in want:
+                wants.setdefault(step, []).append((rid, pos[rid] + w))
+            pos[rid] += n
+        lines.append({"step": step, "entries": entries, "end": []})
+        step += 1
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    # live at most: a 100->128, b 70->128, c 130->192 = 448; later d 64 + c 192 + e 128
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", "448"],
+                          input="\n".join(json.dumps(l) for l in lines) + "\n", capture_output=True, text=True,
+                          timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.split("\n") if l] == [f"done {i}" for i in range(step)]
+    plain_logits = {k: H.plain_logits(folder, v, ROUNDING[dtype]) for k, v in reqs.items()}
+    V = c["cfg"].vocab_size
+    for s, places in wants.items():
+        got = torch.from_numpy(np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(len(places), V))
+        want = torch.stack([plain_logits[rid][p] for rid, p in places])
+        assert H.rel_err(got, want) < TOL[dtype], (s, places)
