@@ -1,0 +1,90 @@
+"""Command line in the manner of the reference's example.py and bench.py: the engine's
+options carry the names of its Config fields (nanovllm/config.py:6-19), the sampling
+options those of SamplingParams (nanovllm/sampling_params.py:4-11).
+
+    python -m nano_vllm_amd.cli generate --model DIR --prompt-ids 1,2,3 [--prompt "text"] ...
+    python -m nano_vllm_amd.cli random-model --config config.json --seed 0 --out DIR
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+
+
+def add_engine_options(ap: argparse.ArgumentParser) -> None:
+    ap.add_argument("--model", required=True, help="folder with config.json and *.safetensors")
+    ap.add_argument("--max-num-batched-tokens", type=int, default=16384)
+    ap.add_argument("--max-num-seqs", type=int, default=512)
+    ap.add_argument("--max-model-len", type=int, default=4096)
+    ap.add_argument("--gpu-memory-utilization", type=float, default=0.9)
+    ap.add_argument("--enforce-eager", action="store_true")
+    ap.add_argument("--kvcache-block-size", type=int, default=256)
+    ap.add_argument("--num-kvcache-blocks", type=int, default=-1)
+    ap.add_argument("--dtype", default=None, choices=[None, "bfloat16", "float32"])
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--schedule", default="prefill_first", choices=["prefill_first", "mixed"])
+    ap.add_argument("--no-prefix-caching", action="store_true")
+
+
+def engine_kwargs(args) -> dict:
+    return dict(max_num_batched_tokens=args.max_num_batched_tokens, max_num_seqs=args.max_num_seqs,
+                max_model_len=args.max_model_len, gpu_memory_utilization=args.gpu_memory_utilization,
+                enforce_eager=args.enforce_eager, kvcache_block_size=args.kvcache_block_size,
+                num_kvcache_blocks=args.num_kvcache_blocks, dtype=args.dtype, seed=args.seed,
+                schedule=args.schedule, enable_prefix_caching=not args.no_prefix_caching)
+
+
+def cmd_generate(args) -> int:
+    from . import LLM, SamplingParams
+    prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids] + list(args.prompt)
+    if not prompts:
+        print("give at least one --prompt-ids or --prompt", file=sys.stderr)
+        return 2
+    llm = LLM(args.model, **engine_kwargs(args))
+    sp = SamplingParams(temperature=args.temperature, max_tokens=args.max_tokens, ignore_eos=args.ignore_eos)
+    outs = llm.generate(prompts, sp, use_tqdm=not args.json)
+    if args.json:
+        print(json.dumps(outs))
+    else:
+        for p, o in zip(prompts, outs):
+            print(f"\nPrompt: {p!r}")
+            print(f"Completion: {o['text']!r}" if o["text"] is not None else f"Completion ids: {o['token_ids']}")
+    return 0
+
+
+def cmd_random_model(args) -> int:
+    from .weights import write_random_model
+    with open(args.config) as f:
+        config = json.load(f)
+    write_random_model(args.out, config, args.seed, std=args.std, norm_std=args.norm_std, dtype=args.dtype)
+    print(f"wrote {args.out}/config.json and {args.out}/model.safetensors")
+    return 0
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="nano_vllm_amd")
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    g = sub.add_parser("generate", help="generate from prompts (example.py of the reference)")
+    add_engine_options(g)
+    g.add_argument("--prompt", action="append", default=[], help="a text prompt (needs the folder's tokenizer)")
+    g.add_argument("--prompt-ids", action="append", default=[], help="a prompt as comma-separated token ids")
+    g.add_argument("--temperature", type=float, default=0.6)
+    g.add_argument("--max-tokens", type=int, default=256)
+    g.add_argument("--ignore-eos", action="store_true")
+    g.add_argument("--json", action="store_true", help="print the outputs as one JSON line")
+    g.set_defaults(fn=cmd_generate)
+    r = sub.add_parser("random-model", help="write a model folder with seeded random weights")
+    r.add_argument("--config", required=True, help="a config.json of the architecture")
+    r.add_argument("--seed", type=int, default=0)
+    r.add_argument("--out", required=True)
+    r.add_argument("--std", type=float, default=0.02)
+    r.add_argument("--norm-std", type=float, default=0.0, help="norm weights are 1 + N(0, this)")
+    r.add_argument("--dtype", default=None, choices=[None, "bfloat16", "float32"])
+    r.set_defaults(fn=cmd_random_model)
+    args = ap.parse_args(argv)
+    return args.fn(args)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

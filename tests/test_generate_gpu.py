@@ -1,0 +1,94 @@
+"""Generation through the Python entry point and the command line on the GPU."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+import helpers as H
+import plain_qwen3 as plain
+from nano_vllm_amd import LLM, SamplingParams
+
+pytestmark = pytest.mark.gpu
+
+
+def _llm(name, dtype, **kw):
+    opts = dict(dtype=dtype, kvcache_block_size=H.CONFIGS[name]["page"], num_kvcache_blocks=64,
+                max_num_batched_tokens=16, max_num_seqs=4)
+    opts.update(kw)
+    return LLM(H.model_folder(name, dtype), **opts)
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_greedy_generation_in_float32_is_the_plain_argmax_chain(name):
+    lens = (5, 11, 17) if name == "a" else (3, 9, 24, 40)
+    prompts = [H.random_tokens(H.CONFIGS[name]["cfg"].vocab_size, n, 100 + n) for n in lens]
+    outs = _llm(name, "float32").generate(prompts, SamplingParams(temperature=0.0, max_tokens=8), use_tqdm=False)
+    cfg, w = plain.read_folder(H.model_folder(name, "float32"))
+    for p, o in zip(prompts, outs):
+        assert o["token_ids"] == plain.greedy_generate(w, cfg, p, 8)
+
+
+def test_greedy_generation_in_bfloat16_follows_the_plain_chain():
+    name = "c"
+    prompts = [H.random_tokens(1000, n, 200 + n) for n in (30, 77, 150)]
+    outs = _llm(name, "bfloat16").generate(prompts, SamplingParams(temperature=0.0, max_tokens=12), use_tqdm=False)
+    cfg, w = plain.read_folder(H.model_folder(name, "bfloat16"))
+    same = total = 0
+    for p, o in zip(prompts, outs):
+        # teacher-forced on the engine's own tokens, so that one flipped near-tie does not
+        # turn every later token: the plain logit of the engine's token must be within the
+        # tolerance of the plain maximum
+        toks = list(p)
+        for t in o["token_ids"]:
+            l = plain.logits(w, cfg, toks, "bfloat16")[-1]
+            assert float(l.max() - l[t]) <= 2e-2 * float(l.abs().max())
+            same += int(int(l.argmax()) == t)
+            total += 1
+            toks.append(t)
+    assert same >= 0.8 * total
+
+
+def test_schedules_and_page_shortage_do_not_change_greedy_tokens():
+    name = "b"
+    prompts = [H.random_tokens(384, n, 300 + n) for n in (3, 9, 24, 40, 33, 33)]
+    prompts[5] = prompts[4][:32] + [1]                      # shares four pages with the one before
+    sp = SamplingParams(temperature=0.0, max_tokens=10)
+    base = [o["token_ids"] for o in _llm(name, "float32", enable_prefix_caching=False).generate(prompts, sp, use_tqdm=False)]
+    for kw in (dict(schedule="mixed"), dict(num_kvcache_blocks=14), dict(num_kvcache_blocks=14, schedule="mixed")):
+        llm = _llm(name, "float32", **kw)
+        assert [o["token_ids"] for o in llm.generate(prompts, sp, use_tqdm=False)] == base, kw
+        llm.runner.cache.check()
+        if "num_kvcache_blocks" in kw:
+            assert llm.scheduler.num_preemptions > 0
+
+
+def test_temperature_sampling_is_reproducible_and_independent_of_the_batch():
+    name = "b"
+    prompts = [H.random_tokens(384, n, 400 + n) for n in (7, 19, 31)]
+    sp = SamplingParams(temperature=0.7, max_tokens=10, seed=3)
+    a = [o["token_ids"] for o in _llm(name, "float32").generate(prompts, sp, use_tqdm=False)]
+    b = [o["token_ids"] for o in _llm(name, "float32", max_num_seqs=1).generate(prompts, sp, use_tqdm=False)]
+    assert a == b
+    c = [o["token_ids"] for o in _llm(name, "float32").generate(prompts, SamplingParams(temperature=0.7, max_tokens=10, seed=4), use_tqdm=False)]
+    assert a != c
+
+
+def test_cache_sized_from_free_memory():
+    llm = LLM(H.model_folder("d", "bfloat16"), gpu_memory_utilization=0.05, max_num_batched_tokens=64, max_num_seqs=4)
+    assert llm.config.num_kvcache_blocks > 0 and llm.config.kvcache_block_size == 256
+    out = llm.generate([[1, 2, 3]], SamplingParams(temperature=0.0, max_tokens=3), use_tqdm=False)
+    assert len(out[0]["token_ids"]) == 3
+
+
+def test_command_line_generates(tmp_path):
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "example.py"), "--model", H.model_folder("b", "float32"),
+                           "--prompt-ids", "5,6,7", "--prompt-ids", "9,8", "--temperature", "0", "--max-tokens", "4",
+                           "--kvcache-block-size", "8", "--num-kvcache-blocks", "16", "--json"],
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    outs = json.loads(proc.stdout.strip().split("\n")[-1])
+    cfg, w = plain.read_folder(H.model_folder("b", "float32"))
+    assert [o["token_ids"] for o in outs] == [plain.greedy_generate(w, cfg, p, 4) for p in ([5, 6, 7], [9, 8])]

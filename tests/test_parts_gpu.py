@@ -1,0 +1,273 @@
+"""Each part alone against the plain implementation's function for it, and a toy mixer with
+state of its own, defined here, that is registered, built, loaded and stepped without a
+change to the package's files."""
+import json
+import os
+
+import pytest
+import torch
+
+import helpers as H
+import plain_qwen3 as plain
+from nano_vllm_amd.cache import CacheGroup, CacheManager
+from nano_vllm_amd.config import register_architecture
+from nano_vllm_amd.engine.batch import StepEntry, build_batch
+from nano_vllm_amd.engine.runner import ModelRunner
+from nano_vllm_amd.parts import (BuildContext, FixedState, LayerCache, LayerRun, LayerSpec, ModelSpec, ParamDecl,
+                                 Part, PartSpec, make_part, register_part)
+from nano_vllm_amd.weights import write_random_model
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+TOL = {"float32": 1e-5, "bfloat16": 2.0 ** -6}
+
+
+def _ctx(dtype, hidden=96, max_position=256):
+    from nano_vllm_amd.kernels import HipKernels
+    return BuildContext(HipKernels(DEV, dtype, quiet=True), torch.device(DEV), dtype, hidden, max_position)
+
+
+def _rand(shape, seed, scale=1.0):
+    return scale * torch.randn(shape, generator=torch.Generator().manual_seed(seed))
+
+
+def _err(got, want):
+    return float((got.float().cpu() - want).abs().max() / want.abs().max())
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_norm_part(dt):
+    dtype = DTYPES[dt]
+    part = make_part("norm", PartSpec("rms_norm", {"dim": 120, "eps": 3e-5}), _ctx(dtype))
+    assert part.param_decls()["weight"].shape == (120,)
+    w = (1 + _rand((120,), 1, 0.1)).to(dtype)
+    part.weights["weight"] = w.to(DEV)
+    x, r = _rand((9, 120), 2).to(dtype), _rand((9, 120), 3).to(dtype)
+    rd = None if dt == "float32" else "bfloat16"
+    assert _err(part.forward(x.to(DEV)), plain.rms_norm(x.float(), w.float(), 3e-5, rd)) < TOL[dt]
+    y, res = part.forward_add(x.to(DEV), r.to(DEV).clone())
+    wy, wr = plain.add_rms_norm(x.float(), r.float(), w.float(), 3e-5, rd)
+    assert _err(y, wy) < TOL[dt] and _err(res, wr) < TOL[dt]
+
+
+def test_position_encoding_part():
+    part = make_part("position_encoding", PartSpec("rotary_neox", {"head_dim": 48, "theta": 5e5, "max_position": 300}),
+                     _ctx(torch.float32))
+    t = part.rotary_table().cpu()
+    ang = plain.rope_angles(48, torch.arange(300), 5e5)
+    assert t.shape == (300, 48)
+    assert float((t[:, :24] - ang.cos()).abs().max()) < 2e-6 and float((t[:, 24:] - ang.sin()).abs().max()) < 2e-6
+    none = make_part("position_encoding", PartSpec("none"), _ctx(torch.float32))
+    assert none.rotary_table() is None
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_feed_forward_part(dt):
+    dtype = DTYPES[dt]
+    part = make_part("feed_forward", PartSpec("swiglu", {"hidden_size": 96, "intermediate_size": 200}), _ctx(dtype))
+    decls = part.param_decls()
+    assert decls["gate_up_proj.weight"].shape == (400, 96)
+    assert [s.name for s in decls["gate_up_proj.weight"].sources] == ["gate_proj.weight", "up_proj.weight"]
+    g, u, d = (_rand(s, i, 0.2).to(dtype) for i, s in enumerate([(200, 96), (200, 96), (96, 200)]))
+    part.weights["gate_up_proj.weight"] = torch.cat([g, u]).to(DEV)
+    part.weights["down_proj.weight"] = d.to(DEV)
+    x = _rand((11, 96), 7).to(dtype)
+    want = plain.feed_forward(x.float(), g.float(), u.float(), d.float(), None if dt == "float32" else "bfloat16")
+    assert _err(part.forward(x.to(DEV)), want) < TOL[dt]
+
+
+def _attention_setup(dtype, window=None, qk_norm=True, heads=6, kv_heads=3, D=32, hidden=96, page=8, pages=12):
+    ctx = _ctx(dtype, hidden)
+    ctx.position_encodings["rope"] = make_part("position_encoding", PartSpec(
+        "rotary_neox", {"head_dim": D, "theta": 1e4, "max_position": 256}), ctx)
+    part = make_part("mixer", PartSpec("attention", {
+        "hidden_size": hidden, "num_heads": heads, "num_kv_heads": kv_heads, "head_dim": D, "qk_norm": qk_norm,
+        "eps": 1e-6, "position_encoding": "rope", "window": window}), ctx)
+    w = {"q_proj.weight": _rand((heads * D, hidden), 1, 0.2), "k_proj.weight": _rand((kv_heads * D, hidden), 2, 0.2),
+         "v_proj.weight": _rand((kv_heads * D, hidden), 3, 0.2), "o_proj.weight": _rand((hidden, heads * D), 4, 0.2),
+         "q_norm.weight": 1 + _rand((D,), 5, 0.1), "k_norm.weight": 1 + _rand((D,), 6, 0.1)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    part.weights["qkv_proj.weight"] = torch.cat([w["q_proj.weight"], w["k_proj.weight"], w["v_proj.weight"]]).to(DEV)
+    part.weights["o_proj.weight"] = w["o_proj.weight"].to(DEV)
+    if qk_norm:
+        part.weights["q_norm.weight"] = w["q_norm.weight"].to(DEV)
+        part.weights["k_norm.weight"] = w["k_norm.weight"].to(DEV)
+    need = part.cache_need()
+    cache = CacheManager([CacheGroup(window, (0,))], page, pages, enable_prefix_caching=False)
+    lc = LayerCache(group=0, k=torch.zeros((pages, need.num_kv_heads, page, need.head_dim), dtype=dtype, device=DEV),
+                    v=torch.zeros((pages, need.num_kv_heads, need.head_dim, page), dtype=dtype, device=DEV))
+    pcfg = plain.PlainConfig(vocab_size=10, hidden_size=hidden, num_layers=1, num_heads=heads, num_kv_heads=kv_heads,
+                             head_dim=D, intermediate_size=1, rms_norm_eps=1e-6, rope_theta=1e4, max_position=256,
+                             tie_word_embeddings=False, attention_bias=False)
+    return part, cache, lc, {f"a.{k}": v.float() for k, v in w.items()}, pcfg
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("window", [None, 10])
+def test_attention_part_in_portions(dt, window):
+    dtype = DTYPES[dt]
+    part, cache, lc, w, pcfg = _attention_setup(dtype, window)
+    assert part.cache_need().window == window
+    T = 60
+    x = _rand((T, 96), 9).to(dtype)
+    rd = None if dt == "float32" else "bfloat16"
+    want = plain.self_attention(x.float(), torch.arange(T), w, "a", pcfg, window, rd)
+    cache.admit("r")
+    got, pos = [], 0
+    for n in (13, 1, 1, 20, 2, 23):
+        cache.reserve("r", pos + n, first_query=pos)
+        batch = build_batch([StepEntry("r", [0] * n, pos, [])], cache, 8, 10, DEV)
+        got.append(part.forward(x[pos:pos + n].to(DEV), batch, lc))
+        pos += n
+        cache.check()
+    assert _err(torch.cat(got), want) < TOL[dt]
+    if window:
+        assert cache.table("r", 0)[0] == -1                  # the window has passed the first pages
+    part.kernels.check_faults()
+
+
+def test_attention_part_without_qk_norm_and_with_bias_declares_its_tensors():
+    ctx = _ctx(torch.float32)
+    part = make_part("mixer", PartSpec("attention", {"hidden_size": 96, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16,
+                                                     "qk_norm": False, "bias": True, "position_encoding": None}), ctx)
+    decls = part.param_decls()
+    assert set(decls) == {"qkv_proj.weight", "qkv_proj.bias", "o_proj.weight"}
+    assert [(s.name, s.row, s.rows) for s in decls["qkv_proj.bias"].sources] == [
+        ("q_proj.bias", 0, 64), ("k_proj.bias", 64, 32), ("v_proj.bias", 96, 32)]
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+def test_block_part(dt):
+    """The pre-norm residual block: first without, then with an incoming residual."""
+    dtype = DTYPES[dt]
+    name = "b"
+    folder = H.model_folder(name, dt)
+    r = H.make_runner(folder, dt, 8, 16)
+    cfg, w = plain.read_folder(folder)
+    rd = None if dt == "float32" else "bfloat16"
+    T = 20
+    toks = H.random_tokens(cfg.vocab_size, T, 3)
+    r.cache.admit("x")
+    r.cache.reserve("x", T)
+    batch = build_batch([StepEntry("x", toks, 0, [])], r.cache, 8, cfg.vocab_size, DEV)
+    h0 = w["model.embed_tokens.weight"][torch.tensor(toks)]
+    pos = torch.arange(T)
+
+    def plain_layer(i, h, res):
+        p = f"model.layers.{i}"
+        if res is None:
+            x, res = plain.rms_norm(h, w[f"{p}.input_layernorm.weight"], cfg.rms_norm_eps, rd), h
+        else:
+            x, res = plain.add_rms_norm(h, res, w[f"{p}.input_layernorm.weight"], cfg.rms_norm_eps, rd)
+        a = plain.self_attention(x, pos, w, f"{p}.self_attn", cfg, None, rd)
+        y, res = plain.add_rms_norm(a, res, w[f"{p}.post_attention_layernorm.weight"], cfg.rms_norm_eps, rd)
+        return plain.feed_forward(y, w[f"{p}.mlp.gate_proj.weight"], w[f"{p}.mlp.up_proj.weight"],
+                                  w[f"{p}.mlp.down_proj.weight"], rd), res
+
+    h = h0.to(dtype).to(DEV)
+    m1, r1 = r.model.blocks[0].forward(h, None, batch, r.layer_caches[0])
+    wm1, wr1 = plain_layer(0, h0, None)
+    assert _err(m1, wm1) < 4 * TOL[dt] and _err(r1, wr1) < TOL[dt]
+    m2, r2 = r.model.blocks[1].forward(m1, r1, batch, r.layer_caches[1])
+    wm2, wr2 = plain_layer(1, wm1, wr1)
+    assert _err(m2, wm2) < 8 * TOL[dt] and _err(r2, wr2) < 4 * TOL[dt]
+
+
+# ------------------------------------------------------------------------------ a toy mixer with state
+class ToyDecayMixer(Part):
+    """s_t = decay * s_{t-1} + x_t per request, kept in a state slot; out_t = s_t W^T.
+    Written with torch operations: a mixer need not use the package's kernels."""
+
+    def __init__(self, params, build):
+        super().__init__(params, build)
+        self.hidden = params["hidden_size"]
+        self.decay = params["decay"]
+
+    def param_decls(self):
+        return {"mix.weight": ParamDecl((self.hidden, self.hidden))}
+
+    def cache_need(self):
+        return FixedState({"s": ((self.hidden,), "float32")})
+
+    def forward(self, x, batch, cache):
+        out = torch.empty_like(x)
+        state = cache.state["s"]
+        slots = batch.state_slots.tolist()
+        t = 0
+        for s, (n, start) in enumerate(zip(batch.q_lens, batch.starts)):
+            cur = torch.zeros(self.hidden, device=x.device) if start == 0 else state[slots[s]].clone()
+            for i in range(n):
+                cur = self.decay * cur + x[t + i].float()
+                out[t + i] = (self.weights["mix.weight"].float() @ cur).to(x.dtype)
+            state[slots[s]] = cur
+            t += n
+        return out
+
+
+def _toy_spec(cfg: dict) -> ModelSpec:
+    H_, V = cfg["hidden_size"], cfg["vocab_size"]
+    norm = PartSpec("rms_norm", {"dim": H_, "eps": cfg["eps"]})
+    ffn = PartSpec("swiglu", {"hidden_size": H_, "intermediate_size": cfg["inner"]})
+    attn = PartSpec("attention", {"hidden_size": H_, "num_heads": 4, "num_kv_heads": 2, "head_dim": 16, "qk_norm": True,
+                                  "eps": cfg["eps"], "position_encoding": "rope", "window": None})
+    toy = PartSpec("toy_decay", {"hidden_size": H_, "decay": cfg["decay"]})
+    names = {"mixer_norm": "norm1", "mixer": "mixer", "feed_forward_norm": "norm2", "feed_forward": "ffn"}
+    layers = tuple(LayerSpec(PartSpec("pre_norm_residual"), {"mixer_norm": norm, "mixer": m, "feed_forward_norm": norm,
+                                                              "feed_forward": ffn}, f"layers.{i}", names)
+                   for i, m in enumerate([toy, attn]))
+    return ModelSpec(architecture="ToyStateLM", hidden_size=H_, vocab_size=V, max_position=128, dtype="float32",
+                     embedding=PartSpec("token_embedding", {"name": "embed"}), layers=layers,
+                     order=(LayerRun(0), LayerRun(1), LayerRun(0)),          # the toy layer runs twice
+                     final_norm=PartSpec("rms_norm", {"dim": H_, "eps": cfg["eps"], "name": "norm"}),
+                     head=PartSpec("output_head", {"name": "head", "tied": True}),
+                     position_encodings={"rope": PartSpec("rotary_neox", {"head_dim": 16, "theta": 1e4, "max_position": 128})})
+
+
+def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
+    register_part("mixer", "toy_decay", ToyDecayMixer, replace=True)
+    register_architecture("ToyStateLM", lambda d: d, _toy_spec, replace=True)
+    cfg = {"architectures": ["ToyStateLM"], "hidden_size": 64, "vocab_size": 99, "inner": 72, "eps": 1e-5, "decay": 0.5,
+           "torch_dtype": "float32"}
+    folder = write_random_model(str(tmp_path / "toy"), cfg, seed=5, std=0.1)
+    r = ModelRunner.from_folder(folder, dtype="float32", page_size=8, num_pages=16, max_requests=3, quiet=True)
+    assert len(r.groups) == 1 and r.state_runs == [0, 2] and r.cache.slots.num_slots == 3
+    assert not r.cache.prefix_caching
+    assert "layers.0.mixer.mix.weight" in r.model.params
+    reqs = {k: H.random_tokens(99, n, i) for i, (k, n) in enumerate({"a": 30, "b": 17, "c": 41}.items())}
+
+    def drive(plan):
+        pos = {k: 0 for k in reqs}
+        got = {k: [] for k in reqs}
+        for k in reqs:
+            r.cache.admit(k)
+        for step in plan:
+            entries = []
+            for k, n in step:
+                r.cache.reserve(k, pos[k] + n)
+                entries.append(StepEntry(k, reqs[k][pos[k]:pos[k] + n], pos[k], list(range(n))))
+                pos[k] += n
+            out = r.step(entries)
+            row = 0
+            for e in entries:
+                got[e.request].append(out[row:row + len(e.tokens)].cpu())
+                row += len(e.tokens)
+        for k in reqs:
+            r.cache.release(k)
+        r.cache.check()
+        return {k: torch.cat(v) for k, v in got.items()}
+
+    whole = drive([[("a", 30)], [("b", 17)], [("c", 41)]])
+    cut = drive([[("a", 7), ("b", 1)], [("c", 20), ("a", 1), ("b", 10)], [("a", 22), ("c", 1)], [("b", 6), ("c", 20)]])
+    for k in reqs:
+        assert H.rel_err(cut[k], whole[k]) < 2e-5, k
+    # the state does its work: a request cut in two without its state differs from the whole
+    r.cache.admit("a")
+    r.cache.reserve("a", 30)
+    r.step([StepEntry("a", reqs["a"][:10], 0, [])])
+    for lc in r.layer_caches:
+        if lc.state is not None:
+            lc.state["s"].zero_()
+    lost = r.step([StepEntry("a", reqs["a"][10:], 10, list(range(20)))]).cpu()
+    r.cache.release("a")
+    assert H.rel_err(lost, whole["a"][10:]) > 1e-3
