@@ -1,0 +1,272 @@
+// Decode attention on the matrix cores (bfloat16): one query token per request against the
+// request's keys in the paged cache, split over the context.
+//
+// Semantics as in attn_generic.hip (nanovllm/layers/attention.py:71-74, causal).  The token at
+// position p reads keys first..p, first = max(0, p - window + 1) with a window, else 0.
+//
+// Work split: one wave per (split of the context, kv head, token).  The G = Hq / Hkv query heads
+// of a kv head share its keys: they are the 16 columns of a 16x16x32 MFMA (columns >= G idle).
+// A wave walks its split in chunks of 32 keys:
+//   S^T[32 keys x 16 heads] = K[32 x D] Q^T          2 tiles x D/32 MFMAs, K rows straight from global
+//   online softmax over keys (in-lane, then across the 4 lane groups)
+//   O^T[D x 16 heads] += V^T[D x 32 keys] P^T        D/16 MFMAs; P stays in registers
+// The transposed V cache [pages, Hkv, D, page] makes 8 consecutive keys of one channel one 16-byte
+// load; the rows of the two S tiles are interleaved (tile a: keys 8g..8g+3, tile b: 8g+4..8g+7 for
+// lane group g) so that a lane's eight probabilities are exactly the eight keys of that load.
+// Each split writes an unnormalised partial result (max, sum, O); a second kernel merges them.
+// With a single split the first kernel writes the result itself.
+//
+// Requires head_dim % 32 == 0 (32..256), G <= 16, page_size % 8 == 0; the launcher refuses
+// anything else and the caller falls back to the general kernel.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define DEC_CHUNK 32
+
+template <int D>
+__global__ void __launch_bounds__(NVA_WAVE)
+attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
+                   float* __restrict__ part_o, float* __restrict__ part_ml,
+                   const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
+                   const int32_t* __restrict__ block_tables, int table_stride,
+                   const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
+                   int num_q_heads, int num_kv_heads, int page_size, float scale, int window, int split_len,
+                   int num_splits, int32_t* error_flag) {
+    constexpr int KP = D / 32;          // 16-byte pieces of a key row per lane = MFMAs per S tile
+    constexpr int DT = D / 16;          // 16-channel tiles of the output
+    const int split = blockIdx.x, kvh = blockIdx.y;
+    const int64_t t = blockIdx.z;
+    const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
+    const int G = num_q_heads / num_kv_heads;
+    const int pos = positions[t];
+    const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    const int kv_len = pos + 1;
+    // the splits are cut at multiples of split_len of the absolute position
+    const int lo = max(split * split_len, first & ~(DEC_CHUNK - 1));
+    const int hi = min((split + 1) * split_len, kv_len);
+    if (lo >= hi) return;
+    const int32_t* table = block_tables + (int64_t)token_seq[t] * table_stride;
+
+    // Q: column `col` is query head kvh*G + col; lane group g holds channels [g*D/4, (g+1)*D/4)
+    bf16x8 qf[KP];
+    {
+        const __bf16* qrow = q + t * q_stride + (int64_t)(kvh * G + (col < G ? col : 0)) * D + g * (D / 4);
+#pragma unroll
+        for (int c = 0; c < KP; ++c) {
+            bf16x8 v = *reinterpret_cast<const bf16x8*>(qrow + 8 * c);
+            if (col >= G) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
+            }
+            qf[c] = v;
+        }
+    }
+
+    f32x4 acc[DT];
+#pragma unroll
+    for (int i = 0; i < DT; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+
+    // row r of S tile a is key 8*(r/4) + r%4 of the chunk, of tile b the same + 4
+    const int row_key = 8 * (col >> 2) + (col & 3);
+
+    for (int base = lo; base < hi; base += DEC_CHUNK) {
+        // ---- K rows of this lane: keys base + row_key (+4), channels of lane group g
+        bf16x8 ka[KP], kb[KP];
+        const int key_a = base + row_key, key_b = key_a + 4;
+        {
+            const bool ok_a = key_a >= first && key_a < kv_len, ok_b = key_b >= first && key_b < kv_len;
+            const int page_a = ok_a ? table[key_a / page_size] : 0;
+            const int page_b = ok_b ? table[key_b / page_size] : 0;
+            if ((ok_a && page_a < 0) || (ok_b && page_b < 0)) {
+                if (error_flag) atomicOr(error_flag, 2);
+            }
+            const __bf16* pa = k_cache + (((int64_t)max(page_a, 0) * num_kv_heads + kvh) * page_size + key_a % page_size) * D + g * (D / 4);
+            const __bf16* pb = k_cache + (((int64_t)max(page_b, 0) * num_kv_heads + kvh) * page_size + key_b % page_size) * D + g * (D / 4);
+#pragma unroll
+            for (int c = 0; c < KP; ++c) {
+                bf16x8 z;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) z[e] = (__bf16)0.f;
+                ka[c] = ok_a ? *reinterpret_cast<const bf16x8*>(pa + 8 * c) : z;
+                kb[c] = ok_b ? *reinterpret_cast<const bf16x8*>(pb + 8 * c) : z;
+            }
+        }
+        // ---- V: channel 16*dt + col, keys base + 8g .. base + 8g + 7 (one page: page_size % 8 == 0)
+        bf16x8 vf[DT];
+        {
+            const int key0 = base + 8 * g;
+            const bool ok = key0 + 8 > first && key0 < kv_len;       // the group holds a visible key
+            const int page = ok ? table[key0 / page_size] : 0;
+            if (ok && page < 0 && error_flag) atomicOr(error_flag, 2);
+            const __bf16* pv = v_cache + (((int64_t)max(page, 0) * num_kv_heads + kvh) * D + col) * (int64_t)page_size + key0 % page_size;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                bf16x8 v;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
+                if (ok) v = *reinterpret_cast<const bf16x8*>(pv + (int64_t)dt * 16 * page_size);
+                if (key0 + 8 > kv_len || key0 < first) {       // the ends of the visible range: drop what lies outside
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        if (key0 + e >= kv_len || key0 + e < first) v[e] = (__bf16)0.f;
+                }
+                vf[dt] = v;
+            }
+        }
+        // ---- scores
+        f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KP; ++c) {
+            sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], qf[c], sa, 0, 0, 0);
+            sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[c], qf[c], sb, 0, 0, 0);
+        }
+        // this lane: head `col`, keys base + 8g + i (tile a) and base + 8g + 4 + i (tile b)
+        float s[8];
+        float m_new = m_run;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int key = base + 8 * g + i;
+            const float v = (i < 4 ? sa[i] : sb[i - 4]) * scale;
+            s[i] = (key >= first && key < kv_len) ? v : -INFINITY;
+            m_new = fmaxf(m_new, s[i]);
+        }
+        m_new = fmaxf(m_new, __shfl_xor(m_new, 16, NVA_WAVE));
+        m_new = fmaxf(m_new, __shfl_xor(m_new, 32, NVA_WAVE));
+        float psum = 0.f;
+        bf16x8 pf;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float p = (s[i] == -INFINITY) ? 0.f : __expf(s[i] - m_new);
+            const __bf16 pb16 = (__bf16)p;
+            pf[i] = pb16;
+            psum += (float)pb16;           // the sum of what the product below really uses
+        }
+        psum += __shfl_xor(psum, 16, NVA_WAVE);
+        psum += __shfl_xor(psum, 32, NVA_WAVE);
+        const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            f32x4 a = acc[dt];
+            a[0] *= alpha; a[1] *= alpha; a[2] *= alpha; a[3] *= alpha;
+            acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pf, a, 0, 0, 0);
+        }
+    }
+
+    // acc[dt][i] = O[head col][channel 16*dt + 4*g + i]
+    if (col >= G) return;
+    const int head = kvh * G + col;
+    if (num_splits == 1) {
+        const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+        __bf16* orow = out + t * out_stride + (int64_t)head * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) orow[16 * dt + 4 * g + i] = (__bf16)(acc[dt][i] * inv);
+    } else {
+        const int64_t slot = ((int64_t)t * num_q_heads + head) * num_splits + split;
+        float* po = part_o + slot * D;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            *reinterpret_cast<f32x4*>(po + 16 * dt + 4 * g) = acc[dt];
+        if (g == 0) {
+            part_ml[slot * 2] = m_run;
+            part_ml[slot * 2 + 1] = l_run;
+        }
+    }
+}
+
+// Merges the splits of one (token, head): o = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m).
+__global__ void __launch_bounds__(NVA_WAVE)
+attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                         __bf16* __restrict__ out, int64_t out_stride, const int32_t* __restrict__ positions,
+                         int num_q_heads, int head_dim, int window, int split_len, int num_splits) {
+    const int64_t t = blockIdx.x;
+    const int head = blockIdx.y, lane = threadIdx.x;
+    const int pos = positions[t];
+    const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    const int s_lo = first / split_len, s_hi = pos / split_len;          // splits that hold visible keys
+    const int64_t slot0 = ((int64_t)t * num_q_heads + head) * num_splits;
+    float m = -INFINITY;
+    for (int s = s_lo; s <= s_hi; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
+    float l = 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = s_lo; s <= s_hi; ++s) {
+        const float ms = part_ml[(slot0 + s) * 2];
+        const float w = (ms == -INFINITY) ? 0.f : __expf(ms - m);
+        l += part_ml[(slot0 + s) * 2 + 1] * w;
+        const float* po = part_o + (slot0 + s) * head_dim;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int d = lane + i * NVA_WAVE;
+            if (d < head_dim) acc[i] += po[d] * w;
+        }
+    }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    __bf16* orow = out + t * out_stride + (int64_t)head * head_dim;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int d = lane + i * NVA_WAVE;
+        if (d < head_dim) orow[d] = (__bf16)(acc[i] * inv);
+    }
+}
+
+// Returns 1 (and leaves a message) for shapes this kernel does not take; the caller then uses the
+// general kernel.  split_len must be a multiple of 32; num_splits = ceil(max kv length / split_len).
+NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride, float* scratch,
+                                    const void* k_cache, const void* v_cache, const int32_t* block_tables,
+                                    int table_stride, const int32_t* token_seq, const int32_t* positions,
+                                    int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
+                                    float scale, int window, int split_len, int num_splits, int32_t* error_flag,
+                                    hipStream_t stream) {
+    if (tokens == 0) return 0;
+    if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
+        return nva_fail("attn_decode: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
+    const int G = num_q_heads / num_kv_heads;
+    if (G > 16 || head_dim % 32 || head_dim < 32 || head_dim > 256 || page_size % 8 || page_size <= 0) {
+        nva_fail("attn_decode: needs head_dim %% 32 == 0 in 32..256, at most 16 query heads per kv head and "
+                 "page_size %% 8 == 0 (got head_dim %d, group %d, page %d)", head_dim, G, page_size);
+        return 1;
+    }
+    if (tokens < 0 || tokens > 65535 || num_kv_heads > 65535)
+        return nva_fail("attn_decode: %lld tokens or %d kv heads exceed the grid", (long long)tokens, num_kv_heads);
+    if (split_len <= 0 || split_len % DEC_CHUNK || num_splits <= 0 || window < 0 || table_stride <= 0)
+        return nva_fail("attn_decode: bad split_len %d / num_splits %d / window %d", split_len, num_splits, window);
+    if (num_splits > 1 && !scratch) return nva_fail("attn_decode: several splits need scratch memory");
+    float* part_o = scratch;
+    float* part_ml = scratch ? scratch + tokens * num_q_heads * (int64_t)num_splits * head_dim : nullptr;
+    dim3 grid((unsigned)num_splits, (unsigned)num_kv_heads, (unsigned)tokens);
+#define LAUNCH(DD)                                                                                              \
+    hipLaunchKernelGGL(attn_decode_kernel<DD>, grid, dim3(NVA_WAVE), 0, stream, (const __bf16*)q, q_stride,       \
+                       (__bf16*)out, out_stride, part_o, part_ml, (const __bf16*)k_cache, (const __bf16*)v_cache, \
+                       block_tables, table_stride, token_seq, positions, num_q_heads, num_kv_heads, page_size,    \
+                       scale, window, split_len, num_splits, error_flag)
+    switch (head_dim) {
+        case 32: LAUNCH(32); break;
+        case 64: LAUNCH(64); break;
+        case 96: LAUNCH(96); break;
+        case 128: LAUNCH(128); break;
+        case 160: LAUNCH(160); break;
+        case 192: LAUNCH(192); break;
+        case 224: LAUNCH(224); break;
+        case 256: LAUNCH(256); break;
+        default: return nva_fail("attn_decode: head_dim %d has no instance", head_dim);
+    }
+#undef LAUNCH
+    int rc = nva_check_launch("attn_decode");
+    if (rc) return rc;
+    if (num_splits > 1) {
+        dim3 mgrid((unsigned)tokens, (unsigned)num_q_heads);
+        hipLaunchKernelGGL(attn_decode_merge_kernel, mgrid, dim3(NVA_WAVE), 0, stream, part_o, part_ml, (__bf16*)out,
+                           out_stride, positions, num_q_heads, head_dim, window, split_len, num_splits);
+        rc = nva_check_launch("attn_decode_merge");
+    }
+    return rc;
+}
+
+NVA_DEFINE_LAST_ERROR(nva_attn_decode)

@@ -66,6 +66,8 @@ class HipKernels:
         self.fault_flag = torch.zeros(1, dtype=torch.int32, device=self.device)
         # Rows up to which the bfloat16 product runs on the engine's own kernels.
         self.own_matmul_rows = 0
+        # False: attention always runs the general kernel (tests compare the two)
+        self.mfma_attention = True
 
     # ------------------------------------------------------------------ helpers
     def _stream(self):
@@ -267,11 +269,47 @@ class HipKernels:
         _, ow, os_ = _rows2d(out, "attention out")
         if ow != width or out.shape[0] != tokens or out.dtype != q.dtype:
             raise KernelError("attention: output does not match q")
-        library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q), c_i64(qs), _p(out), c_i64(os_),
-                     _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.token_seq),
-                     _p(batch.positions), c_i64(tokens), c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim),
-                     c_i32(page_size), c_f32(scale), c_i32(window or 0), _p(self.fault_flag), self._stream())
+        # tokens [0, num_decode) are single decoded tokens: the matrix-core decode kernel takes
+        # them where its shape limits allow; everything else runs the general kernel
+        start = 0
+        if q.dtype == torch.bfloat16 and batch.num_decode > 0 and self.mfma_attention and \
+                self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
+            start = batch.num_decode
+            self._attention_decode(q, qs, out, os_, k_cache, v_cache, tables, batch, start, num_heads, num_kv_heads,
+                                   head_dim, page_size, scale, window)
+        if start < tokens:
+            n = tokens - start
+            library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q[start:]), c_i64(qs),
+                         _p(out[start:]), c_i64(os_), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
+                         _p(batch.token_seq[start:]), _p(batch.positions[start:]), c_i64(n), c_i32(num_heads),
+                         c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
+                         _p(self.fault_flag), self._stream())
         return out
+
+    @staticmethod
+    def _decode_kernel_takes(group, head_dim, page_size, q, q_stride, out, out_stride) -> bool:
+        return (group <= 16 and head_dim % 32 == 0 and 32 <= head_dim <= 256 and page_size % 8 == 0
+                and q.data_ptr() % 16 == 0 and q_stride % 8 == 0 and out.data_ptr() % 16 == 0 and out_stride % 8 == 0)
+
+    def _attention_decode(self, q, qs, out, os_, k_cache, v_cache, tables, batch, n, num_heads, num_kv_heads,
+                          head_dim, page_size, scale, window):
+        max_kv = batch.max_kv_len
+        split_len = 64
+        for cand in (8192, 4096, 2048, 1024, 512, 256, 128):       # the longest split that still fills the GPU
+            if n * num_kv_heads * ((max_kv + cand - 1) // cand) >= 2048:
+                split_len = cand
+                break
+        num_splits = (max_kv + split_len - 1) // split_len
+        scratch = None
+        if num_splits > 1:
+            scratch = torch.empty(n * num_heads * num_splits * (head_dim + 2), dtype=torch.float32, device=q.device)
+        for t0 in range(0, n, 65535):                               # grid.z holds at most 65535 tokens
+            t1 = min(n, t0 + 65535)
+            library.call("attn_decode", "bf16", "nva_attn_decode", _p(q[t0:t1]), c_i64(qs), _p(out[t0:t1]), c_i64(os_),
+                         _p(scratch), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
+                         _p(batch.token_seq[t0:t1]), _p(batch.positions[t0:t1]), c_i64(t1 - t0), c_i32(num_heads),
+                         c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
+                         c_i32(split_len), c_i32(num_splits), _p(self.fault_flag), self._stream())
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:
