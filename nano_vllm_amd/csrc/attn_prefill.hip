@@ -1,0 +1,272 @@
+// Prefill attention on the matrix cores (bfloat16): portions of prompts against the paged cache.
+//
+// Semantics as in attn_generic.hip (nanovllm/layers/attention.py:64-70: causal, the diagonal
+// aligned to the end of the keys when a request has cached tokens before this step's).  A request
+// with q_len new tokens and kv_len tokens in the cache after this step has its query i at position
+// kv_len - q_len + i; it reads keys first..position, first = max(0, position - window + 1) with a
+// window, else 0.  The step's own keys are in the cache already.
+//
+// Work split: a workgroup of 4 waves takes 32 query rows of one request and up to 4 query heads of
+// one kv head (one head per wave), so that a K/V tile is fetched once for the group.  Per tile of
+// 64 keys, staged in LDS from the pages (K rows, and V rows of the transposed V cache):
+//   S^T[64 keys x 32 queries] = K Q^T                 32x32x16 MFMAs, Q in registers
+//   online softmax per query column (in-lane + one exchange between the lane halves)
+//   O^T[D x 32 queries] += V^T P^T                    P never leaves registers
+// The rows of the S tiles are permuted (row 8a+4h+b holds key 16(a/2)+8h+4(a%2)+b) so that the
+// sixteen scores a lane holds per tile are keys 8h..8h+7 and 16+8h..16+8h+7: two operands of the
+// second product as they are.
+//
+// Requires head_dim % 32 == 0 (32..256) and page_size % 8 == 0; the launcher refuses anything else
+// and the caller falls back to the general kernel.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+#define PF_BM 32
+#define PF_BN 64
+#define PF_WAVES 4
+
+template <int D>
+__global__ void __launch_bounds__(PF_WAVES * NVA_WAVE)
+attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
+                    const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
+                    const int32_t* __restrict__ block_tables, int table_stride,
+                    const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens, int first_seq,
+                    int num_seqs, int num_q_heads, int num_kv_heads, int page_size, float scale, int window,
+                    int32_t* error_flag) {
+    constexpr int KS = D + 8;             // K tile row stride (elements): 16 bytes of padding against bank conflicts
+    constexpr int VS = PF_BN + 8;         // V tile row stride
+    constexpr int DC = D / 16;            // 16-channel steps of the first product
+    constexpr int MT = D / 32;            // 32-channel tiles of the output
+    __shared__ __attribute__((aligned(16))) __bf16 k_s[PF_BN * KS];
+    __shared__ __attribute__((aligned(16))) __bf16 v_s[D * VS];
+
+    // ---- which request and which 32 rows of it
+    int seq = first_seq, tile = blockIdx.x;
+    for (; seq < num_seqs; ++seq) {
+        const int tiles = (cu_seqlens_q[seq + 1] - cu_seqlens_q[seq] + PF_BM - 1) / PF_BM;
+        if (tile < tiles) break;
+        tile -= tiles;
+    }
+    if (seq >= num_seqs) return;
+    const int q_begin = cu_seqlens_q[seq];
+    const int q_len = cu_seqlens_q[seq + 1] - q_begin;
+    const int kv_len = kv_lens[seq];
+    const int start = kv_len - q_len;                 // position of the request's first query of this step
+    const int q0 = tile * PF_BM;
+    const int32_t* table = block_tables + (int64_t)seq * table_stride;
+
+    const int G = num_q_heads / num_kv_heads;
+    const int chunks = (G + PF_WAVES - 1) / PF_WAVES;
+    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int tid = threadIdx.x, wave = tid / NVA_WAVE, lane = tid % NVA_WAVE;
+    const int col = lane & 31, h = lane >> 5;
+    const int head_in_group = chunk * PF_WAVES + wave;
+    const bool active = head_in_group < G;
+    const int head = kvh * G + (active ? head_in_group : 0);
+
+    const int row = q0 + col;                         // this lane's query row within the request's portion
+    const bool row_ok = row < q_len;
+    const int pos = start + row;
+
+    // keys any row of the tile may see
+    const int last_pos = start + min(q0 + PF_BM, q_len) - 1;
+    const int first_any = window > 0 && start + q0 - window + 1 > 0 ? start + q0 - window + 1 : 0;
+    const int kb_lo = first_any & ~(PF_BN - 1);
+    const int kb_hi = last_pos + 1;                   // exclusive
+
+    // ---- Q: column = query row, lane half h holds channels 16c + 8h .. + 7
+    bf16x8 qf[DC];
+    {
+        const __bf16* qrow = q + (int64_t)(q_begin + (row_ok ? row : 0)) * q_stride + (int64_t)head * D + 8 * h;
+#pragma unroll
+        for (int c = 0; c < DC; ++c) {
+            bf16x8 v = *reinterpret_cast<const bf16x8*>(qrow + 16 * c);
+            if (!row_ok || !active) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
+            }
+            qf[c] = v;
+        }
+    }
+
+    f32x16 acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][e] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    // S tile row r = col holds key 16*(a/2) + 8*h' + 4*(a%2) + b with a = r/8, h' = (r/4)%2, b = r%4
+    const int a_r = col >> 3, h_r = (col >> 2) & 1, b_r = col & 3;
+    const int row_key = 16 * (a_r >> 1) + 8 * h_r + 4 * (a_r & 1) + b_r;
+    const int first_row = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+
+    for (int kb = kb_lo; kb < kb_hi; kb += PF_BN) {
+        // ---- stage the K tile: 64 rows of D channels
+        for (int idx = tid; idx < PF_BN * (D / 8); idx += PF_WAVES * NVA_WAVE) {
+            const int r = idx / (D / 8), piece = idx % (D / 8);
+            const int key = kb + r;
+            bf16x8 v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
+            if (key >= first_any && key < kb_hi) {
+                const int page = table[key / page_size];
+                if (page < 0) {
+                    if (error_flag) atomicOr(error_flag, 2);
+                } else {
+                    v = *reinterpret_cast<const bf16x8*>(
+                        k_cache + (((int64_t)page * num_kv_heads + kvh) * page_size + key % page_size) * D + piece * 8);
+                }
+            }
+            *reinterpret_cast<bf16x8*>(&k_s[r * KS + piece * 8]) = v;
+        }
+        // ---- stage the V tile: D rows of 64 keys (8 keys = 16 bytes lie in one page)
+        for (int idx = tid; idx < D * (PF_BN / 8); idx += PF_WAVES * NVA_WAVE) {
+            const int d = idx / (PF_BN / 8), grp = idx % (PF_BN / 8);
+            const int key0 = kb + grp * 8;
+            bf16x8 v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
+            if (key0 + 8 > first_any && key0 < kb_hi) {
+                const int page = table[key0 / page_size];
+                if (page < 0) {
+                    if (error_flag) atomicOr(error_flag, 2);
+                } else {
+                    v = *reinterpret_cast<const bf16x8*>(
+                        v_cache + (((int64_t)page * num_kv_heads + kvh) * D + d) * (int64_t)page_size + key0 % page_size);
+                    if (key0 + 8 > kb_hi || key0 < first_any) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (key0 + e >= kb_hi || key0 + e < first_any) v[e] = (__bf16)0.f;
+                    }
+                }
+            }
+            *reinterpret_cast<bf16x8*>(&v_s[d * VS + grp * 8]) = v;
+        }
+        __syncthreads();
+
+        if (active) {
+            // ---- scores of 2 x 32 keys
+            f32x16 s[2];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s[kt][e] = 0.f;
+                const __bf16* krow = &k_s[(kt * 32 + row_key) * KS + 8 * h];
+#pragma unroll
+                for (int c = 0; c < DC; ++c) {
+                    const bf16x8 a = *reinterpret_cast<const bf16x8*>(krow + 16 * c);
+                    s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], s[kt], 0, 0, 0);
+                }
+            }
+            // this lane: query `col`; register e of tile kt is key kb + 32*kt + 16*(e/8) + 8*h + e%8
+            const bool full = kb + PF_BN - 1 <= start + q0 && kb >= first_any + (window > 0 ? PF_BM : 0);
+            float m_new = m_run;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float v = s[kt][e] * scale;
+                    if (!full) {
+                        const int key = kb + 32 * kt + 16 * (e >> 3) + 8 * h + (e & 7);
+                        if (key > pos || key < first_row) v = -INFINITY;
+                    }
+                    s[kt][e] = v;
+                    m_new = fmaxf(m_new, v);
+                }
+            m_new = fmaxf(m_new, __shfl_xor(m_new, 32, NVA_WAVE));
+            float psum = 0.f;
+            bf16x8 pf[2][2];
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float p = (s[kt][e] == -INFINITY) ? 0.f : __expf(s[kt][e] - m_new);
+                    const __bf16 pb = (__bf16)p;
+                    pf[kt][e >> 3][e & 7] = pb;
+                    psum += (float)pb;
+                }
+            psum += __shfl_xor(psum, 32, NVA_WAVE);
+            const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                f32x16 o = acc[mt];
+#pragma unroll
+                for (int e = 0; e < 16; ++e) o[e] *= alpha;
+                const __bf16* vrow = &v_s[(mt * 32 + col) * VS + 8 * h];
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int ks = 0; ks < 2; ++ks) {
+                        const bf16x8 a = *reinterpret_cast<const bf16x8*>(vrow + kt * 32 + ks * 16);
+                        o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[kt][ks], o, 0, 0, 0);
+                    }
+                acc[mt] = o;
+            }
+        }
+        __syncthreads();
+    }
+
+    // acc[mt][4a + b] = O[query col][channel 32*mt + 8a + 4h + b]
+    if (!active || !row_ok) return;
+    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    __bf16* orow = out + (int64_t)(q_begin + row) * out_stride + (int64_t)head * D;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            bf16x4 v;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) v[b] = (__bf16)(acc[mt][4 * a + b] * inv);
+            *reinterpret_cast<bf16x4*>(orow + 32 * mt + 8 * a + 4 * h) = v;
+        }
+}
+
+// total_tiles = sum over requests first_seq.. of ceil(q_len / 32), computed by the caller.
+// Returns 1 (and leaves a message) for shapes this kernel does not take.
+NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride,
+                                     const void* k_cache, const void* v_cache, const int32_t* block_tables,
+                                     int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
+                                     int first_seq, int num_seqs, int64_t total_tiles, int num_q_heads,
+                                     int num_kv_heads, int head_dim, int page_size, float scale, int window,
+                                     int32_t* error_flag, hipStream_t stream) {
+    if (total_tiles == 0 || first_seq >= num_seqs) return 0;
+    if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
+        return nva_fail("attn_prefill: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
+    if (head_dim % 32 || head_dim < 32 || head_dim > 256 || page_size % 8 || page_size <= 0) {
+        nva_fail("attn_prefill: needs head_dim %% 32 == 0 in 32..256 and page_size %% 8 == 0 (got %d, %d)", head_dim,
+                 page_size);
+        return 1;
+    }
+    const int G = num_q_heads / num_kv_heads;
+    const int64_t grid_y = (int64_t)num_kv_heads * ((G + PF_WAVES - 1) / PF_WAVES);
+    if (total_tiles < 0 || total_tiles > 0x7fffffff || grid_y > 65535 || window < 0 || table_stride <= 0)
+        return nva_fail("attn_prefill: bad sizes (tiles %lld, heads %lld)", (long long)total_tiles, (long long)grid_y);
+    dim3 grid((unsigned)total_tiles, (unsigned)grid_y);
+#define LAUNCH(DD)                                                                                                 \
+    hipLaunchKernelGGL(attn_prefill_kernel<DD>, grid, dim3(PF_WAVES * NVA_WAVE), 0, stream, (const __bf16*)q,        \
+                       q_stride, (__bf16*)out, out_stride, (const __bf16*)k_cache, (const __bf16*)v_cache,           \
+                       block_tables, table_stride, cu_seqlens_q, kv_lens, first_seq, num_seqs, num_q_heads,          \
+                       num_kv_heads, page_size, scale, window, error_flag)
+    switch (head_dim) {
+        case 32: LAUNCH(32); break;
+        case 64: LAUNCH(64); break;
+        case 96: LAUNCH(96); break;
+        case 128: LAUNCH(128); break;
+        case 160: LAUNCH(160); break;
+        case 192: LAUNCH(192); break;
+        case 224: LAUNCH(224); break;
+        case 256: LAUNCH(256); break;
+        default: return nva_fail("attn_prefill: head_dim %d has no instance", head_dim);
+    }
+#undef LAUNCH
+    return nva_check_launch("attn_prefill");
+}
+
+NVA_DEFINE_LAST_ERROR(nva_attn_prefill)

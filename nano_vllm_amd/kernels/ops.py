@@ -269,6 +269,8 @@ class HipKernels:
         _, ow, os_ = _rows2d(out, "attention out")
         if ow != width or out.shape[0] != tokens or out.dtype != q.dtype:
             raise KernelError("attention: output does not match q")
+        if any(n != 1 for n in batch.q_lens[:batch.num_decode]):
+            raise KernelError("attention: the first num_decode requests of a batch must bring one token each")
         # tokens [0, num_decode) are single decoded tokens: the matrix-core decode kernel takes
         # them where its shape limits allow; everything else runs the general kernel
         start = 0
@@ -277,6 +279,16 @@ class HipKernels:
             start = batch.num_decode
             self._attention_decode(q, qs, out, os_, k_cache, v_cache, tables, batch, start, num_heads, num_kv_heads,
                                    head_dim, page_size, scale, window)
+        if start < tokens and q.dtype == torch.bfloat16 and self.mfma_attention and start == batch.num_decode and \
+                self._decode_kernel_takes(1, head_dim, page_size, q, qs, out, os_):
+            # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
+            tiles = sum((n + 31) // 32 for n in batch.q_lens[batch.num_decode:])
+            library.call("attn_prefill", "bf16", "nva_attn_prefill", _p(q), c_i64(qs), _p(out), c_i64(os_), _p(k_cache),
+                         _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q), _p(batch.kv_lens),
+                         c_i32(batch.num_decode), c_i32(batch.num_seqs), c_i64(tiles), c_i32(num_heads),
+                         c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
+                         _p(self.fault_flag), self._stream())
+            start = tokens
         if start < tokens:
             n = tokens - start
             library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q[start:]), c_i64(qs),

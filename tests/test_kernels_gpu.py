@@ -229,7 +229,7 @@ def _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed, boost=None):
         positions=torch.tensor(positions, dtype=torch.int32, device=DEV), max_kv_len=max(lens), max_q_len=max(q_lens),
         kv_lens=torch.tensor(lens, dtype=torch.int32, device=DEV),
         cu_seqlens_q=torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=DEV),
-        num_decode=sum(1 for n in q_lens if n == 1), q_lens=list(q_lens),
+        num_decode=next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens)), q_lens=list(q_lens),
         groups=[SimpleNamespace(block_tables=tables.to(DEV), slot_mapping=None)])
     return q, kc, vc, batch, (qs, ks, vs)
 
@@ -252,6 +252,10 @@ ATT_CASES = [
     (7, 1, 64, 32, [90, 31], [45, 1], None),                       # seven heads on one kv head
     (4, 2, 128, 16, [200, 50], [30, 1], 24),                       # window
     (2, 1, 256, 8, [33], [33], 5),
+    (8, 2, 128, 64, [300, 500, 77, 130], [1, 1, 77, 100], None),   # the shape of a served step
+    (4, 4, 64, 16, [1, 2, 3, 40], [1, 2, 3, 40], None),            # the first tokens of requests
+    (16, 1, 32, 8, [70, 9], [1, 9], None),                         # sixteen heads on one kv head
+    (3, 1, 96, 24, [150, 100], [1, 100], 40),                      # a window over pages of 24
 ]
 
 
@@ -266,6 +270,13 @@ def test_paged_attention(hip, ref, dtype, hq, hkv, D, page, lens, q_lens, window
     twin = ref.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window)
     _close(got, twin, dtype, "against the plain paged attention")
     hip[dtype].check_faults()
+    if dtype == torch.bfloat16:
+        # the general kernel in bfloat16 (the fallback of shapes the matrix-core kernels refuse)
+        hip[dtype].mfma_attention = False
+        try:
+            _close(hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window), twin, dtype, "general")
+        finally:
+            hip[dtype].mfma_attention = True
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
