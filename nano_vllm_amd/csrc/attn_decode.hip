@@ -182,6 +182,8 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 }
 
 // Merges the splits of one (token, head): o = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m).
+// One wave per (token, head).  The (max, sum) pairs of up to 64 splits are read by 64 lanes at
+// once; the partial outputs are then read four splits at a time so that the loads overlap.
 __global__ void __launch_bounds__(NVA_WAVE)
 attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                          __bf16* __restrict__ out, int64_t out_stride, const int32_t* __restrict__ positions,
@@ -193,20 +195,42 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
     const int s_lo = first / split_len, s_hi = pos / split_len;          // splits that hold visible keys
     const int64_t slot0 = ((int64_t)t * num_q_heads + head) * num_splits;
     float m = -INFINITY;
-    for (int s = s_lo; s <= s_hi; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
+    for (int s0 = s_lo; s0 <= s_hi; s0 += NVA_WAVE) {
+        const int s = s0 + lane;
+        m = fmaxf(m, s <= s_hi ? part_ml[(slot0 + s) * 2] : -INFINITY);
+    }
+    m = wave_max(m);
     float l = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s = s_lo; s <= s_hi; ++s) {
-        const float ms = part_ml[(slot0 + s) * 2];
-        const float w = (ms == -INFINITY) ? 0.f : __expf(ms - m);
-        l += part_ml[(slot0 + s) * 2 + 1] * w;
-        const float* po = part_o + (slot0 + s) * head_dim;
+    for (int s0 = s_lo; s0 <= s_hi; s0 += NVA_WAVE) {
+        const int s = s0 + lane;
+        float w = 0.f;
+        if (s <= s_hi) {
+            const float ms = part_ml[(slot0 + s) * 2];
+            w = (ms == -INFINITY) ? 0.f : __expf(ms - m);
+            l += part_ml[(slot0 + s) * 2 + 1] * w;
+        }
+        const int count = min(NVA_WAVE, s_hi - s0 + 1);
+        for (int j0 = 0; j0 < count; j0 += 4) {
+            float wj[4], v[4][4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int d = lane + i * NVA_WAVE;
-            if (d < head_dim) acc[i] += po[d] * w;
+            for (int j = 0; j < 4; ++j) {
+                wj[j] = __shfl(w, min(j0 + j, NVA_WAVE - 1), NVA_WAVE);
+                if (j0 + j >= count) wj[j] = 0.f;
+                const float* po = part_o + (slot0 + s0 + min(j0 + j, count - 1)) * head_dim;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = lane + i * NVA_WAVE;
+                    v[j][i] = d < head_dim ? po[d] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] += v[j][i] * wj[j];
         }
     }
+    l = wave_sum(l);
     const float inv = l > 0.f ? 1.f / l : 0.f;
     __bf16* orow = out + t * out_stride + (int64_t)head * head_dim;
 #pragma unroll

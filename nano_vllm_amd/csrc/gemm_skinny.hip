@@ -1,0 +1,196 @@
+// y[M, N] = x[M, K] W[N, K]^T for few rows (M <= 16, bfloat16): the linear layers of a decode
+// step (nanovllm/layers/linear.py:51,73,153; embed_head.py:61), where every weight is read once
+// and the time is the time to stream W from HBM.
+//
+// One wave owns 16 output columns (16 rows of W) over a range of k.  W rows are the A operand of
+// a 16x16x32 MFMA, the rows of x its 16 columns (rows >= M idle).  A lane reads 64 contiguous bytes of its W row per step of 128 k
+// (the k index is permuted alike in both operands), straight from global into registers; the
+// workgroup's slice of x is staged in LDS.  For small N the k range is split over workgroups, each
+// writing float partial sums; a second kernel adds the partials in a fixed order, applies the
+// optional bias and the optional SwiGLU gating (W = [gate rows; up rows]) and rounds once.
+//
+// Requires K % 8 == 0 and 16-byte aligned rows; the launcher refuses anything else and the caller
+// uses the library product or the tiled kernel.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+#define SK_WAVES 4
+#define SK_KSTEP 128
+#define SK_UNROLL 2
+#define SK_CHUNK 1536     // k of x staged at a time: 16 rows * (1536 + 8) * 2 bytes of LDS
+
+__device__ __forceinline__ bf16x8 zero8() {
+    bf16x8 z;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) z[e] = (__bf16)0.f;
+    return z;
+}
+
+// direct: 1 = the only split writes y itself (as bfloat16 or float); 0 = float partials [split][M][N]
+//
+// The workgroup's four waves share one range of k, so its slice of x (16 rows, rows >= M zero) is
+// staged once in LDS (row stride padded by 16 bytes against bank conflicts).  The loads of the next
+// step's W fragments are issued before the products of the current one.
+__global__ void __launch_bounds__(SK_WAVES * NVA_WAVE)
+linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf16* __restrict__ w, int64_t w_stride,
+                     float* __restrict__ partial, void* __restrict__ y, int64_t y_stride, int y_is_f32, int direct,
+                     int M, int N, int K, int k_per_split) {
+    extern __shared__ __attribute__((aligned(16))) __bf16 x_s[];     // [16][chunk + 8]
+    const int wave = threadIdx.x / NVA_WAVE, lane = threadIdx.x % NVA_WAVE;
+    const int col = lane & 15, g = lane >> 4;
+    const int split = blockIdx.y;
+    const int k_begin = split * k_per_split;
+    const int k_end = min(K, k_begin + k_per_split);
+    const int chunk = min(k_per_split, SK_CHUNK);
+    const int xs_stride = chunk + 8;
+
+    const int n0 = (blockIdx.x * SK_WAVES + wave) * 16;
+    const bool active = n0 < N;                       // idle waves still help to stage x
+    const int wrow = min(n0 + col, N - 1);
+    const __bf16* wp = w + (int64_t)wrow * w_stride + 32 * g;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+
+    for (int c_begin = k_begin; c_begin < k_end; c_begin += chunk) {
+        const int c_end = min(k_end, c_begin + chunk);
+        // ---- stage x[0:16][c_begin:c_begin + chunk] (zeros beyond M and c_end)
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < 16 * (chunk / 8); idx += SK_WAVES * NVA_WAVE) {
+            const int m = idx / (chunk / 8), piece = idx % (chunk / 8);
+            const int k = c_begin + piece * 8;
+            bf16x8 v = zero8();
+            if (m < M && k < c_end) v = *reinterpret_cast<const bf16x8*>(x + (int64_t)m * x_stride + k);
+            *reinterpret_cast<bf16x8*>(&x_s[m * xs_stride + piece * 8]) = v;
+        }
+        __syncthreads();
+        if (!active) continue;
+        const __bf16* xp = x_s + col * xs_stride + 32 * g - c_begin;
+
+        bf16x8 a_next[SK_UNROLL][4];
+#pragma unroll
+        for (int u = 0; u < SK_UNROLL; ++u)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int k = c_begin + u * SK_KSTEP + 32 * g + 8 * c;
+                a_next[u][c] = k < c_end ? *reinterpret_cast<const bf16x8*>(wp + c_begin + u * SK_KSTEP + 8 * c) : zero8();
+            }
+        for (int kk = c_begin; kk < c_end; kk += SK_KSTEP * SK_UNROLL) {
+            bf16x8 a[SK_UNROLL][4];
+#pragma unroll
+            for (int u = 0; u < SK_UNROLL; ++u)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) a[u][c] = a_next[u][c];
+            const int kn = kk + SK_KSTEP * SK_UNROLL;
+            if (kn < c_end) {
+#pragma unroll
+                for (int u = 0; u < SK_UNROLL; ++u)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const int k = kn + u * SK_KSTEP + 32 * g + 8 * c;
+                        a_next[u][c] = k < c_end ? *reinterpret_cast<const bf16x8*>(wp + kn + u * SK_KSTEP + 8 * c) : zero8();
+                    }
+            }
+#pragma unroll
+            for (int u = 0; u < SK_UNROLL; ++u) {
+                if (kk + u * SK_KSTEP < c_end) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        // x_s holds zeros beyond c_end, up to the padded end of the chunk
+                        const bf16x8 b = *reinterpret_cast<const bf16x8*>(xp + kk + u * SK_KSTEP + 8 * c);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][c], b, acc, 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+    if (!active) return;
+    // acc[i] = y[m = col][n = n0 + 4*g + i]
+    const int n = n0 + 4 * g;
+    const int m = col;
+    if (m >= M) return;
+    if (!direct) {
+        float* p = partial + ((int64_t)split * M + m) * N + n;
+        if (n + 3 < N && (N % 4) == 0) {
+            *reinterpret_cast<f32x4*>(p) = acc;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n + i < N) p[i] = acc[i];
+        }
+    } else if (y_is_f32) {
+        float* p = (float*)y + (int64_t)m * y_stride + n;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (n + i < N) p[i] = acc[i];
+    } else {
+        __bf16* p = (__bf16*)y + (int64_t)m * y_stride + n;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (n + i < N) p[i] = (__bf16)acc[i];
+    }
+}
+
+// y[m][n] = sum over splits of partial[s][m][n] (+ bias[n]); with swiglu, N is the width of the
+// partials (2 * inner) and y[m][j] = silu(sum_gate[j]) * sum_up[j], j < inner.
+__global__ void __launch_bounds__(256)
+linear_skinny_finish_kernel(const float* __restrict__ partial, int splits, const __bf16* __restrict__ bias,
+                            void* __restrict__ y, int64_t y_stride, int y_is_f32, int swiglu, int M, int N) {
+    const int out_n = swiglu ? N / 2 : N;
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)M * out_n) return;
+    const int m = (int)(idx / out_n), j = (int)(idx % out_n);
+    float v = 0.f, u = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float* p = partial + ((int64_t)s * M + m) * N;
+        v += p[j];
+        if (swiglu) u += p[out_n + j];
+    }
+    if (bias) {
+        v += (float)bias[j];
+        if (swiglu) u += (float)bias[out_n + j];
+    }
+    if (swiglu) {
+        // the reference rounds the projection to bfloat16 before the gating (activation.py:8-11)
+        v = (float)(__bf16)v;
+        u = (float)(__bf16)u;
+        v = v / (1.f + __expf(-v)) * u;
+    }
+    if (y_is_f32) ((float*)y)[(int64_t)m * y_stride + j] = v;
+    else ((__bf16*)y)[(int64_t)m * y_stride + j] = (__bf16)v;
+}
+
+// splits: how many ranges k is cut into (>= 1); scratch must hold splits * M * N floats when
+// splits > 1 or a bias or swiglu is asked for.  Returns 1 for shapes this kernel does not take.
+NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
+                                      const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
+                                      float* scratch, int splits, int64_t M, int64_t N, int64_t K,
+                                      hipStream_t stream) {
+    if (M == 0 || N == 0) return 0;
+    if (M < 0 || M > 16 || K % 8 || K <= 0 || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
+        nva_fail("linear_skinny: needs 1..16 rows, K %% 8 == 0 and 16-byte aligned rows (M=%lld K=%lld)", (long long)M,
+                 (long long)K);
+        return 1;
+    }
+    if (N > 0x7fffffff || K > 0x7fffffff || splits < 1 || splits > 65535) return nva_fail("linear_skinny: bad sizes");
+    if (swiglu && (N % 2)) return nva_fail("linear_skinny: the gated form needs an even number of weight rows");
+    const int direct = splits == 1 && !bias && !swiglu;
+    if (!direct && !scratch) return nva_fail("linear_skinny: this call needs scratch memory");
+    int kps = (int)((K + splits - 1) / splits);
+    kps = (kps + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
+    const int real_splits = (int)((K + kps - 1) / kps);
+    const int64_t tiles = (N + 15) / 16;
+    dim3 grid((unsigned)((tiles + SK_WAVES - 1) / SK_WAVES), (unsigned)real_splits);
+    const size_t lds = (size_t)16 * ((kps < SK_CHUNK ? kps : SK_CHUNK) + 8) * sizeof(__bf16);
+    hipLaunchKernelGGL(linear_skinny_kernel, grid, dim3(SK_WAVES * NVA_WAVE), lds, stream, (const __bf16*)x, x_stride,
+                       (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32, direct, (int)M, (int)N, (int)K, kps);
+    int rc = nva_check_launch("linear_skinny");
+    if (rc || direct) return rc;
+    const int64_t outs = M * (swiglu ? N / 2 : N);
+    hipLaunchKernelGGL(linear_skinny_finish_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, stream, scratch,
+                       real_splits, (const __bf16*)bias, y, y_stride, y_is_f32, swiglu, (int)M, (int)N);
+    return nva_check_launch("linear_skinny_finish");
+}
+
+NVA_DEFINE_LAST_ERROR(nva_gemm_skinny)

@@ -50,9 +50,15 @@ class StepBatch:
     requests: List[Hashable] = field(default_factory=list)
 
 
-def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size: int, device) -> StepBatch:
+def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size: int, device,
+                table_width: Optional[int] = None, static: Optional[torch.Tensor] = None) -> StepBatch:
     """Orders the entries (single tokens first), checks them against the cache manager's
-    block tables and uploads everything in one copy."""
+    block tables and uploads everything in one copy.
+
+    table_width fixes the width of the block tables (else: the widest table of the batch).
+    static, an int32 device tensor of the batch's flat size, receives the copy instead of a
+    new tensor: with equal counts of tokens, requests and wanted places and a fixed table
+    width the layout is the same for every step, which is what a captured graph replays on."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
@@ -109,13 +115,24 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
             rows.append(offsets[i] + w)
 
     widths = [max(1, max(len(tb) for tb in tables[g])) for g in range(num_groups)]
+    if table_width is not None:
+        if max(widths, default=1) > table_width:
+            raise ValueError(f"a block table of {max(widths)} pages exceeds the fixed width {table_width}")
+        widths = [table_width] * num_groups
     flat: List[int] = []
     flat += input_ids + positions + token_seq + cu + kv_lens + starts + state_slots + rows
     for g in range(num_groups):
         flat += slot_maps[g]
         for tb in tables[g]:
             flat += tb + [-1] * (widths[g] - len(tb))
-    dev = torch.tensor(flat, dtype=torch.int32).to(device)
+    host = torch.tensor(flat, dtype=torch.int32)
+    if static is not None:
+        if static.numel() != host.numel():
+            raise ValueError("the static batch buffer does not fit this batch's layout")
+        static.copy_(host)
+        dev = static
+    else:
+        dev = host.to(device)
 
     pos = 0
 

@@ -41,6 +41,8 @@ class LLMEngine:
             cfg.num_kvcache_blocks = num_pages
         self.runner = ModelRunner(self.model, cfg.kvcache_block_size, num_pages, cfg.max_num_seqs,
                                   enable_prefix_caching=cfg.enable_prefix_caching)
+        if not cfg.enforce_eager and self.model.device.type == "cuda":
+            self.runner.enable_decode_graphs(min(cfg.max_num_seqs, 512), cfg.max_model_len)
         eos = [cfg.eos] if cfg.eos >= 0 else list(spec.eos_token_ids) or self._eos_from_generation_config()
         self.tokenizer = None
         self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens,

@@ -38,6 +38,9 @@ class ModelRunner:
                                   has_state=bool(self.state_runs), enable_prefix_caching=enable_prefix_caching)
         self.layer_caches = storage.allocate(self.needs, self.groups, self.state_runs, counts, page_size,
                                              max_requests, model.dtype, self.device)
+        self._graphs = {}
+        self._graph_max_batch = 0
+        self._graph_max_len = 0
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -52,12 +55,67 @@ class ModelRunner:
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Runs the entries' tokens as one batch.  Their pages must be reserved in
         self.cache.  Returns float32 logits [wanted places, vocab] in the order of the
-        entries and of their `want`, or None if nothing is wanted."""
+        entries and of their `want`, or None if nothing is wanted.  (With decode graphs
+        enabled the tensor returned for a pure decode step is overwritten by the next such
+        step of the same batch size.)"""
+        if self._graph_max_batch and self._graph_takes(entries):
+            return self._step_graph(entries)
         batch = build_batch(entries, self.cache, self.page_size, self.model.spec.vocab_size, self.device)
         hidden = self.model.forward(batch, self.layer_caches)
         if batch.logits_rows is None:
             return None
         return self.model.logits(hidden, batch.logits_rows)
+
+    # ------------------------------------------------------------------ captured decode steps
+    def enable_decode_graphs(self, max_batch: int, max_len: int) -> None:
+        """Decode steps (one token per request, its logits wanted) of up to max_batch requests
+        and max_len cached tokens are captured as HIP graphs, one per batch size, at their
+        first occurrence, and replayed from then on.  Reference: capture_cudagraph and the
+        replay branch of run_model (nanovllm/engine/model_runner.py:195-212,222-257), which
+        pads to a few sizes instead."""
+        if self.state_runs:
+            return          # a mixer with host-side state handling cannot be replayed blindly
+        self._graph_max_batch = max_batch
+        self._graph_max_len = max_len
+        self._graph_table_width = (max_len + self.page_size - 1) // self.page_size
+
+    def _graph_takes(self, entries) -> bool:
+        if len(entries) > self._graph_max_batch or self.device.type != "cuda":
+            return False
+        for e in entries:
+            if len(e.tokens) != 1 or len(e.want) != 1 or e.want[0] != 0 or e.start + 1 > self._graph_max_len:
+                return False
+        return True
+
+    def _step_graph(self, entries) -> torch.Tensor:
+        n = len(entries)
+        vocab = self.model.spec.vocab_size
+        g = self._graphs.get(n)
+        if g is None:
+            # the flat layout of n single tokens with every logit wanted and tables of fixed width
+            num_groups = len(self.groups)
+            size = 3 * n + (n + 1) + 3 * n + n + num_groups * (n + n * self._graph_table_width)
+            static = torch.zeros(size, dtype=torch.int32, device=self.device)
+            batch = build_batch(entries, self.cache, self.page_size, vocab, self.device,
+                                table_width=self._graph_table_width, static=static)
+            batch.max_kv_len = self._graph_max_len        # launch shapes must cover every later step
+            side = torch.cuda.Stream(self.device)
+            side.wait_stream(torch.cuda.current_stream(self.device))
+            with torch.cuda.stream(side):                 # what is set up lazily is set up outside the capture
+                for _ in range(2):
+                    self.model.logits(self.model.forward(batch, self.layer_caches), batch.logits_rows)
+            torch.cuda.current_stream(self.device).wait_stream(side)
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = self.model.logits(self.model.forward(batch, self.layer_caches), batch.logits_rows)
+            g = (graph, static, logits)
+            self._graphs[n] = g
+        graph, static, logits = g
+        build_batch(entries, self.cache, self.page_size, vocab, self.device,
+                    table_width=self._graph_table_width, static=static)
+        graph.replay()
+        return logits
 
 
 def load_model(folder: str, dtype: Optional[str] = None, device="cuda:0", kernels=None, quiet: bool = False) -> Model:

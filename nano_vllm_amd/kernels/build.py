@@ -30,6 +30,7 @@ MODULES: Dict[str, Tuple[str, Tuple[Optional[str], ...]]] = {
     "rope": ("rope.hip", ("bf16", "f32")),
     "attn_generic": ("attn_generic.hip", ("bf16", "f32")),
     "gemm": ("gemm.hip", ("bf16", "f32")),
+    "gemm_skinny": ("gemm_skinny.hip", ("bf16",)),
     "attn_decode": ("attn_decode.hip", ("bf16",)),
     "attn_prefill": ("attn_prefill.hip", ("bf16",)),
     "sample": ("sample.hip", (None,)),

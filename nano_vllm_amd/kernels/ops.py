@@ -65,7 +65,7 @@ class HipKernels:
         # bit 0: a token id outside the vocabulary; bit 1: a visible key without a page
         self.fault_flag = torch.zeros(1, dtype=torch.int32, device=self.device)
         # Rows up to which the bfloat16 product runs on the engine's own kernels.
-        self.own_matmul_rows = 0
+        self.own_matmul_rows = 16
         # False: attention always runs the general kernel (tests compare the two)
         self.mfma_attention = True
 
@@ -168,7 +168,18 @@ class HipKernels:
         if bias is not None and (bias.shape != (n,) or bias.dtype != x.dtype or not bias.is_contiguous()):
             raise KernelError("linear: bias does not fit")
         out_dtype = torch.float32 if out_float32 else x.dtype
-        if x.dtype == torch.bfloat16 and not out_float32 and m > self.own_matmul_rows:
+        if x.dtype == torch.bfloat16 and self._skinny_takes(x, xs, weight, ws, k):
+            if m <= self.own_matmul_rows or out_float32:
+                if out is None:
+                    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+                om, on, os_ = _rows2d(out, "linear output")
+                if (om, on) != (m, n) or out.dtype != out_dtype:
+                    raise KernelError("linear: output does not match")
+                for r0 in range(0, m, 16):          # more rows (logits of many places): 16 at a time
+                    r1 = min(m, r0 + 16)
+                    self._linear_skinny(x[r0:r1], xs, weight, ws, bias, out[r0:r1], os_, out_float32, False, r1 - r0, n, k)
+                return out
+        if x.dtype == torch.bfloat16 and not out_float32:
             y = torch.nn.functional.linear(x, weight, bias)
             if out is not None:
                 out.copy_(y)
@@ -184,8 +195,30 @@ class HipKernels:
                      c_i64(m), c_i64(n), c_i64(k), self._stream())
         return out
 
+    @staticmethod
+    def _skinny_takes(x, xs, weight, ws, k) -> bool:
+        return k % 8 == 0 and xs % 8 == 0 and ws % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+
+    def _linear_skinny(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k):
+        """The weight-streaming kernel for at most 16 rows; k is split over workgroups when the
+        output is too narrow to fill the GPU."""
+        tiles = (n + 15) // 16
+        splits = max(1, min((2048 + tiles - 1) // tiles, k // 256))
+        direct = splits == 1 and bias is None and not swiglu
+        scratch = None if direct else torch.empty(splits * m * n, dtype=torch.float32, device=x.device)
+        library.call("gemm_skinny", "bf16", "nva_linear_skinny", _p(x), c_i64(xs), _p(weight), c_i64(ws), _p(bias),
+                     _p(out), c_i64(os_), c_i32(1 if out_float32 else 0), c_i32(1 if swiglu else 0), _p(scratch),
+                     c_i32(splits), c_i64(m), c_i64(n), c_i64(k), self._stream())
+
     def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         """silu(x @ Wg.T) * (x @ Wu.T) with weight = [Wg; Wu]."""
+        m, k, xs = _rows2d(x, "linear input")
+        n, wk, ws = _rows2d(weight, "linear weight")
+        if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
+                0 < m <= self.own_matmul_rows and self._skinny_takes(x, xs, weight, ws, k):
+            out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
+            self._linear_skinny(x, xs, weight, ws, None, out, n // 2, False, True, m, n, k)
+            return out
         return self.silu_mul(self.linear(x, weight))
 
     # ------------------------------------------------------------------ position encoding

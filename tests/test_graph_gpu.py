@@ -1,0 +1,60 @@
+"""Captured decode steps: every replay is compared with the same step run eagerly, with the
+program's own eager work (prompt portions of other requests, a changed batch) and
+synchronisations between the replays."""
+import pytest
+import torch
+
+import helpers as H
+from nano_vllm_amd.engine.batch import StepEntry
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["b", "d"])
+def test_graph_replays_equal_eager_steps(name, dtype):
+    c = H.CONFIGS[name]
+    folder = H.model_folder(name, dtype)
+    eager = H.make_runner(folder, dtype, c["page"], 64)
+    graphed = H.make_runner(folder, dtype, c["page"], 64)
+    graphed.enable_decode_graphs(max_batch=8, max_len=c["cfg"].max_position_embeddings)
+    V = c["cfg"].vocab_size
+    reqs = {f"r{i}": H.random_tokens(V, n, 80 + i) for i, n in enumerate((70, 60, 55))}
+    extra = H.random_tokens(V, 37, 99)
+    pos = {}
+    for r in (eager, graphed):
+        for rid, toks in reqs.items():
+            r.cache.admit(rid)
+            r.cache.reserve(rid, 20)
+            r.step([StepEntry(rid, toks[:20], 0, [])])
+    for rid in reqs:
+        pos[rid] = 20
+    live = list(reqs)
+    for step in range(24):
+        if step == 9:
+            live = live[:2]                     # the batch size changes: another graph
+        if step == 15:
+            live = list(reqs)
+        outs = []
+        for r in (eager, graphed):
+            entries = []
+            for rid in live:
+                r.cache.reserve(rid, pos[rid] + 1)
+                entries.append(StepEntry(rid, [reqs[rid][pos[rid]]], pos[rid], [0]))
+            outs.append(r.step(entries).clone())
+            if step % 4 == 1:                   # eager work between the replays: a prompt portion
+                r.cache.admit("x")
+                r.cache.reserve("x", len(extra))
+                r.step([StepEntry("x", extra, 0, [len(extra) - 1])])
+                r.cache.release("x")
+            torch.cuda.synchronize()
+        for rid in live:
+            pos[rid] += 1
+        if dtype == "float32":
+            assert torch.equal(outs[0], outs[1]), f"replay {step} differs from the eager step"
+        else:
+            assert H.rel_err(outs[1], outs[0]) < 1e-5, f"replay {step} differs from the eager step"
+    assert sorted(graphed._graphs) == [2, 3]
+    want = H.plain_logits(folder, reqs["r0"][:pos["r0"]], None if dtype == "float32" else "bfloat16")
+    assert H.rel_err(outs[1][0].cpu(), want[-1]) < (2e-5 if dtype == "float32" else 2e-2)
+    graphed.kernels.check_faults()

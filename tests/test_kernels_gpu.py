@@ -136,6 +136,30 @@ def test_linear_bfloat16(hip, ref, m, n, k):
     _close(hip[torch.bfloat16].linear(x, w), ref.linear(x, w), torch.bfloat16)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (8, 6144, 4096), (64, 320, 12288), (17, 1000, 264), (33, 24, 8),
+                                   (5, 130, 72)])
+def test_linear_bfloat16_few_rows_streams_the_weights(hip, ref, m, n, k):
+    """The decode-step product (few rows, k split over workgroups) against a double product."""
+    x, w = _rand((m, k), torch.bfloat16, 21), _rand((n, k), torch.bfloat16, 22, 0.05)
+    want = x.double() @ w.double().T
+    bound = (x.double().abs() @ w.double().abs().T) * (math.sqrt(k) * 2.0 ** -23) + 1e-30
+    got32 = hip[torch.bfloat16].linear(x, w, out_float32=True)
+    assert bool(((got32.double() - want).abs() <= bound).all())
+    got = hip[torch.bfloat16].linear(x, w)
+    assert got.dtype == torch.bfloat16
+    _close(got, want.float().to(torch.bfloat16), torch.bfloat16)
+    b = _rand((n,), torch.bfloat16, 23)
+    _close(hip[torch.bfloat16].linear(x, w, b), (want + b.double()).float().to(torch.bfloat16), torch.bfloat16)
+
+
+@pytest.mark.parametrize("m,inner,k", [(1, 12288, 4096), (8, 200, 96), (64, 160, 256), (100, 64, 128)])
+def test_linear_silu_mul(hip, ref, m, inner, k):
+    x, w = _rand((m, k), torch.bfloat16, 24), _rand((2 * inner, k), torch.bfloat16, 25, 0.1)
+    _close(hip[torch.bfloat16].linear_silu_mul(x, w), ref.linear_silu_mul(x, w), torch.bfloat16)
+    xf, wf = x.float(), w.float()
+    _close(hip[torch.float32].linear_silu_mul(xf, wf), ref.linear_silu_mul(xf, wf), torch.float32)
+
+
 # ------------------------------------------------------------------------------ rotation and cache write
 def _inv_freq(D, theta):
     return (1.0 / (theta ** (torch.arange(0, D, 2, dtype=torch.float) / D))).to(DEV)
