@@ -1,10 +1,11 @@
 """Device tensors of the cache: for every run of the model's order that keeps keys and
-values, K [pages, kv_heads, page, head_dim] and V [pages, kv_heads, head_dim, page] of its
-group's page count; for every run with fixed state, its tensors [slots, ...].
+values, K [pages, kv_heads, page, head_dim] and V [pages, kv_heads, page / vt, head_dim, vt]
+of its group's page count; for every run with fixed state, its tensors [slots, ...].
 
 Reference: nanovllm/engine/model_runner.py:103-121 keeps one tensor [2, layers, pages,
-page, kv_heads, head_dim].  Here a (page, kv head) tile is contiguous, and V is stored
-transposed so that the keys of one channel are contiguous for the attention kernels.
+page, kv_heads, head_dim].  Here a (page, kv head) block is contiguous, and V is stored
+transposed, in tiles of vt keys, so that the keys of one channel are contiguous for the
+attention kernels (kernels.ops.v_cache_shape).
 """
 from __future__ import annotations
 
@@ -12,6 +13,7 @@ from typing import List, Sequence
 
 import torch
 
+from ..kernels.ops import v_cache_shape
 from ..parts.model import LayerCache, torch_dtype
 
 
@@ -43,7 +45,8 @@ def allocate(needs, groups, state_runs, num_pages: Sequence[int], page_size: int
         for r in group.runs:
             need = needs[r]
             k = torch.zeros((num_pages[g], need.num_kv_heads, page_size, need.head_dim), dtype=dtype, device=device)
-            v = torch.zeros((num_pages[g], need.num_kv_heads, need.head_dim, page_size), dtype=dtype, device=device)
+            v = torch.zeros(v_cache_shape(num_pages[g], need.num_kv_heads, need.head_dim, page_size), dtype=dtype,
+                            device=device)
             caches[r] = LayerCache(group=g, k=k, v=v)
     for r in state_runs:
         caches[r] = LayerCache(state={

@@ -10,8 +10,8 @@
 //   S^T[32 keys x 16 heads] = K[32 x D] Q^T          2 tiles x D/32 MFMAs, K rows straight from global
 //   online softmax over keys (in-lane, then across the 4 lane groups)
 //   O^T[D x 16 heads] += V^T[D x 32 keys] P^T        D/16 MFMAs; P stays in registers
-// The transposed V cache [pages, Hkv, D, page] makes 8 consecutive keys of one channel one 16-byte
-// load; the rows of the two S tiles are interleaved (tile a: keys 8g..8g+3, tile b: 8g+4..8g+7 for
+// The transposed V cache (tiles [D, 32 keys], common.h) makes 8 consecutive keys of one channel one
+// 16-byte load and a chunk's values one contiguous block; the rows of the two S tiles are interleaved (tile a: keys 8g..8g+3, tile b: 8g+4..8g+7 for
 // lane group g) so that a lane's eight probabilities are exactly the eight keys of that load.
 // Each split writes an unnormalised partial result (max, sum, O); a second kernel merges them.
 // With a single split the first kernel writes the result itself.
@@ -24,6 +24,44 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 #define DEC_CHUNK 32
+
+// One chunk of 32 keys for one lane: its two K rows (keys base + row_key and + 4, the channels of
+// lane group g) and, per 16-channel tile, eight consecutive keys of channel `col` of V.  Every load
+// is unconditional: a key outside [first, kv_len) is replaced by the nearest visible one, so that
+// no loaded value has to pass through a select (which would make each load wait for the one
+// before).  What such lanes hold is masked where it is used: scores by the key index, and V in the
+// chunks at the two ends of the visible range.
+template <int D>
+__device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf16x8* vf,
+                                           const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
+                                           int table_window, int window_page0, int first, int kv_len, int num_kv_heads,
+                                           int kvh, int page_size, int row_key, int col, int g, int32_t* error_flag) {
+    constexpr int KP = D / 32, DT = D / 16;
+    const int key_a = min(max(base + row_key, first), kv_len - 1);
+    const int key_b = min(max(base + row_key + 4, first), kv_len - 1);
+    // the group of 8 keys of V, moved to the nearest group that holds a visible key
+    const int key0 = min(max(base + 8 * g, first & ~7), (kv_len - 1) & ~7);
+    // block table entries come from the wave's register window (lane i holds page window_page0 + i)
+    const int page_a = __shfl(table_window, (key_a / page_size - window_page0) & (NVA_WAVE - 1), NVA_WAVE);
+    const int page_b = __shfl(table_window, (key_b / page_size - window_page0) & (NVA_WAVE - 1), NVA_WAVE);
+    const int page_v = __shfl(table_window, (key0 / page_size - window_page0) & (NVA_WAVE - 1), NVA_WAVE);
+    if (page_a < 0 || page_b < 0 || page_v < 0) {
+        if (error_flag) atomicOr(error_flag, 2);
+    }
+    const __bf16* pa = k_cache + (((int64_t)max(page_a, 0) * num_kv_heads + kvh) * page_size + key_a % page_size) * D + g * (D / 4);
+    const __bf16* pb = k_cache + (((int64_t)max(page_b, 0) * num_kv_heads + kvh) * page_size + key_b % page_size) * D + g * (D / 4);
+#pragma unroll
+    for (int c = 0; c < KP; ++c) {
+        ka[c] = *reinterpret_cast<const bf16x8*>(pa + 8 * c);
+        kb[c] = *reinterpret_cast<const bf16x8*>(pb + 8 * c);
+    }
+    // V: channel 16*dt + col, keys key0 .. key0 + 7 (one page: page_size % 8 == 0)
+    const int vt = nva_v_tile(page_size);           // a multiple of 8: the group lies in one tile
+    const __bf16* pv = v_cache + ((int64_t)max(page_v, 0) * num_kv_heads + kvh) * D * (int64_t)page_size +
+                       nva_v_offset(key0 % page_size, col, D, vt);
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) vf[dt] = *reinterpret_cast<const bf16x8*>(pv + (int64_t)dt * 16 * vt);
+}
 
 template <int D>
 __global__ void __launch_bounds__(NVA_WAVE)
@@ -72,49 +110,39 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     // row r of S tile a is key 8*(r/4) + r%4 of the chunk, of tile b the same + 4
     const int row_key = 8 * (col >> 2) + (col & 3);
 
+    // The loads of chunk i + 1 are issued before the products of chunk i, so that a wave always has
+    // a chunk (16 KiB at head_dim 128) in flight.
+    // Lane i of the wave keeps block table entry window_page0 + i: a split spans at most 64 pages
+    // (the launcher checks it), so no chunk needs the table again.
+    const int last_page = (kv_len - 1) / page_size;
+    const int window_page0 = lo / page_size;
+    const int table_window = window_page0 + lane <= last_page ? table[window_page0 + lane] : -1;
+    // The loads of the next chunk are issued, unconditionally, before the products of the current
+    // one (after the last chunk the same chunk is read once more and dropped): one path through the
+    // loop, so that the wait before the products covers exactly the current chunk's loads.
+    const int last_base = lo + ((hi - lo - 1) / DEC_CHUNK) * DEC_CHUNK;
+    bf16x8 ka_n[KP], kb_n[KP], vf_n[DT];
+    load_chunk<D>(lo, ka_n, kb_n, vf_n, k_cache, v_cache, table_window, window_page0, first, kv_len, num_kv_heads, kvh,
+                  page_size, row_key, col, g, error_flag);
     for (int base = lo; base < hi; base += DEC_CHUNK) {
-        // ---- K rows of this lane: keys base + row_key (+4), channels of lane group g
-        bf16x8 ka[KP], kb[KP];
-        const int key_a = base + row_key, key_b = key_a + 4;
-        {
-            const bool ok_a = key_a >= first && key_a < kv_len, ok_b = key_b >= first && key_b < kv_len;
-            const int page_a = ok_a ? table[key_a / page_size] : 0;
-            const int page_b = ok_b ? table[key_b / page_size] : 0;
-            if ((ok_a && page_a < 0) || (ok_b && page_b < 0)) {
-                if (error_flag) atomicOr(error_flag, 2);
-            }
-            const __bf16* pa = k_cache + (((int64_t)max(page_a, 0) * num_kv_heads + kvh) * page_size + key_a % page_size) * D + g * (D / 4);
-            const __bf16* pb = k_cache + (((int64_t)max(page_b, 0) * num_kv_heads + kvh) * page_size + key_b % page_size) * D + g * (D / 4);
+        bf16x8 ka[KP], kb[KP], vf[DT];
 #pragma unroll
-            for (int c = 0; c < KP; ++c) {
-                bf16x8 z;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) z[e] = (__bf16)0.f;
-                ka[c] = ok_a ? *reinterpret_cast<const bf16x8*>(pa + 8 * c) : z;
-                kb[c] = ok_b ? *reinterpret_cast<const bf16x8*>(pb + 8 * c) : z;
-            }
+        for (int c = 0; c < KP; ++c) {
+            ka[c] = ka_n[c];
+            kb[c] = kb_n[c];
         }
-        // ---- V: channel 16*dt + col, keys base + 8g .. base + 8g + 7 (one page: page_size % 8 == 0)
-        bf16x8 vf[DT];
-        {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) vf[dt] = vf_n[dt];
+        load_chunk<D>(min(base + DEC_CHUNK, last_base), ka_n, kb_n, vf_n, k_cache, v_cache, table_window, window_page0,
+                      first, kv_len, num_kv_heads, kvh, page_size, row_key, col, g, error_flag);
+        if (base < first || base + DEC_CHUNK > kv_len) {
+            // a chunk at an end of the visible range: what V holds outside the range may be anything
             const int key0 = base + 8 * g;
-            const bool ok = key0 + 8 > first && key0 < kv_len;       // the group holds a visible key
-            const int page = ok ? table[key0 / page_size] : 0;
-            if (ok && page < 0 && error_flag) atomicOr(error_flag, 2);
-            const __bf16* pv = v_cache + (((int64_t)max(page, 0) * num_kv_heads + kvh) * D + col) * (int64_t)page_size + key0 % page_size;
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                bf16x8 v;
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
-                if (ok) v = *reinterpret_cast<const bf16x8*>(pv + (int64_t)dt * 16 * page_size);
-                if (key0 + 8 > kv_len || key0 < first) {       // the ends of the visible range: drop what lies outside
-#pragma unroll
-                    for (int e = 0; e < 8; ++e)
-                        if (key0 + e >= kv_len || key0 + e < first) v[e] = (__bf16)0.f;
-                }
-                vf[dt] = v;
-            }
+                for (int e = 0; e < 8; ++e)
+                    if (key0 + e >= kv_len || key0 + e < first) vf[dt][e] = (__bf16)0.f;
         }
         // ---- scores
         f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
@@ -261,6 +289,8 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
         return nva_fail("attn_decode: %lld tokens or %d kv heads exceed the grid", (long long)tokens, num_kv_heads);
     if (split_len <= 0 || split_len % DEC_CHUNK || num_splits <= 0 || window < 0 || table_stride <= 0)
         return nva_fail("attn_decode: bad split_len %d / num_splits %d / window %d", split_len, num_splits, window);
+    if (split_len / page_size + 2 > NVA_WAVE)
+        return nva_fail("attn_decode: a split of %d keys spans more than %d pages of %d", split_len, NVA_WAVE - 2, page_size);
     if (num_splits > 1 && !scratch) return nva_fail("attn_decode: several splits need scratch memory");
     float* part_o = scratch;
     float* part_ml = scratch ? scratch + tokens * num_q_heads * (int64_t)num_splits * head_dim : nullptr;

@@ -10,7 +10,7 @@
 // positions j <= p (and j > p - window if window > 0) through the request's block table:
 // s_j = scale * <q, k_j>, P = softmax(s), o = sum_j P_j v_j.  The step's own keys are in the
 // cache already when this runs.
-// Layouts: K [pages, Hkv, page, D], V [pages, Hkv, D, page].  One wave per (token, q head).
+// Layouts: K [pages, Hkv, page, D], V transposed in tiles of keys (common.h).  One wave per (token, q head).
 #include "common.h"
 
 #define ATT_MAX_D 512
@@ -46,6 +46,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
     for (int i = 0; i < ATT_ACC; ++i) acc[i] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
     const bool vec = head_dim % 8 == 0;
+    const int vt = nva_v_tile(page_size);
 
     for (int base = first; base <= pos; base += NVA_WAVE) {
         const int j = base + lane;
@@ -59,7 +60,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
             } else {
                 const int64_t head_base = (int64_t)page * num_kv_heads + kvh;
                 const T* krow = k_cache + (head_base * page_size + off) * head_dim;
-                v_off = head_base * head_dim * (int64_t)page_size + off;
+                v_off = head_base * head_dim * (int64_t)page_size + nva_v_offset(off, 0, head_dim, vt);
                 float dot = 0.f;
                 if (vec) {
                     for (int d = 0; d < head_dim; d += 8) {
@@ -91,7 +92,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, int64_t q_stride, T* __r
             const int d = lane + i * NVA_WAVE;
             if (d < head_dim) {
                 float a = acc[i] * correction;
-                const T* vcol = v_cache + (int64_t)d * page_size;
+                const T* vcol = v_cache + (int64_t)d * vt;
                 for (int jj = 0; jj < valid; ++jj) {
                     const float pj = p_s[jj];
                     if (pj != 0.f) a += pj * to_float(vcol[v_off_s[jj]]);

@@ -58,6 +58,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     const int q0 = tile * PF_BM;
     const int32_t* table = block_tables + (int64_t)seq * table_stride;
 
+    const int vt = nva_v_tile(page_size);
     const int G = num_q_heads / num_kv_heads;
     const int chunks = (G + PF_WAVES - 1) / PF_WAVES;
     const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
@@ -136,7 +137,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                     if (error_flag) atomicOr(error_flag, 2);
                 } else {
                     v = *reinterpret_cast<const bf16x8*>(
-                        v_cache + (((int64_t)page * num_kv_heads + kvh) * D + d) * (int64_t)page_size + key0 % page_size);
+                        v_cache + ((int64_t)page * num_kv_heads + kvh) * D * (int64_t)page_size +
+                        nva_v_offset(key0 % page_size, d, D, vt));
                     if (key0 + 8 > kb_hi || key0 < first_any) {
 #pragma unroll
                         for (int e = 0; e < 8; ++e)

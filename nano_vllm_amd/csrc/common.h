@@ -128,3 +128,61 @@ __device__ __forceinline__ float nva_exp(float x) {
     return __expf(x);
 #endif
 }
+
+// ---------------------------------------------------------------------------- split products
+// A product whose k range was split over workgroups leaves float partial sums
+// [splits][rows][width] (gemm_skinny.hip).  Kernels that consume such a product add the partials
+// in the order of the splits, add the optional bias and round to the element type: what the
+// product's own finishing pass would have stored.
+struct PartialInput {
+    const float* sums;        // null: x is read as elements
+    int splits;
+    int64_t split_stride;     // rows * width
+    const void* bias;         // elements, or null
+};
+
+template <typename T>
+__device__ __forceinline__ float partial_value(const PartialInput& p, int64_t row, int width, int i) {
+    float v = 0.f;
+    const float* q = p.sums + row * width + i;
+#pragma unroll 8
+    for (int s = 0; s < p.splits; ++s) v += q[s * p.split_stride];      // independent loads, one sum in split order
+    if (p.bias) v += to_float(static_cast<const T*>(p.bias)[i]);
+    return round_through<T>(v);
+}
+
+template <typename T>
+__device__ __forceinline__ void partial_value8(const PartialInput& p, int64_t row, int width, int i, float* out) {
+    const float* q = p.sums + row * width + i;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = 0.f;
+#pragma unroll 4
+    for (int s = 0; s < p.splits; ++s) {
+        float v[8];
+        load8(q + s * p.split_stride, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] += v[e];
+    }
+    if (p.bias) {
+        float b[8];
+        load8(static_cast<const T*>(p.bias) + i, b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] += b[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = round_through<T>(out[e]);
+}
+
+
+// ---------------------------------------------------------------------------- cache layout
+// K [pages, kv_heads, page_size, head_dim].
+// V [pages, kv_heads, page_size / vt, head_dim, vt]: transposed (the keys of one channel are
+// contiguous) in tiles of vt keys, vt = 32 when the page size is a multiple of 32, else the page
+// size.  A tile of 32 keys is what the decode attention reads per step: 8 KiB contiguous at
+// head_dim 128, instead of half of every 128-byte line of a whole page.
+__host__ __device__ __forceinline__ int nva_v_tile(int page_size) { return page_size % 32 == 0 ? 32 : page_size; }
+
+// Offset of (key `kip` of the page, channel d) within the [head_dim * page_size] block of one (page, kv head).
+__device__ __forceinline__ int64_t nva_v_offset(int kip, int d, int head_dim, int vt) {
+    return ((int64_t)(kip / vt) * head_dim + d) * vt + kip % vt;
+}

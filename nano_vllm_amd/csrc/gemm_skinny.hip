@@ -162,11 +162,12 @@ linear_skinny_finish_kernel(const float* __restrict__ partial, int splits, const
 }
 
 // splits: how many ranges k is cut into (>= 1); scratch must hold splits * M * N floats when
-// splits > 1 or a bias or swiglu is asked for.  Returns 1 for shapes this kernel does not take.
+// splits > 1 or a bias, swiglu or defer_finish is asked for.  splits_used receives the number of
+// ranges really used (k per range is rounded up to a multiple of 128).  Returns 1 for shapes this kernel does not take.
 NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
                                       const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
-                                      float* scratch, int splits, int64_t M, int64_t N, int64_t K,
-                                      hipStream_t stream) {
+                                      float* scratch, int splits, int defer_finish, int64_t M, int64_t N,
+                                      int64_t K, int* splits_used, hipStream_t stream) {
     if (M == 0 || N == 0) return 0;
     if (M < 0 || M > 16 || K % 8 || K <= 0 || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
         nva_fail("linear_skinny: needs 1..16 rows, K %% 8 == 0 and 16-byte aligned rows (M=%lld K=%lld)", (long long)M,
@@ -175,7 +176,7 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     }
     if (N > 0x7fffffff || K > 0x7fffffff || splits < 1 || splits > 65535) return nva_fail("linear_skinny: bad sizes");
     if (swiglu && (N % 2)) return nva_fail("linear_skinny: the gated form needs an even number of weight rows");
-    const int direct = splits == 1 && !bias && !swiglu;
+    const int direct = splits == 1 && !bias && !swiglu && !defer_finish;
     if (!direct && !scratch) return nva_fail("linear_skinny: this call needs scratch memory");
     int kps = (int)((K + splits - 1) / splits);
     kps = (kps + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
@@ -185,11 +186,26 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     const size_t lds = (size_t)16 * ((kps < SK_CHUNK ? kps : SK_CHUNK) + 8) * sizeof(__bf16);
     hipLaunchKernelGGL(linear_skinny_kernel, grid, dim3(SK_WAVES * NVA_WAVE), lds, stream, (const __bf16*)x, x_stride,
                        (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32, direct, (int)M, (int)N, (int)K, kps);
+    if (splits_used) *splits_used = real_splits;
     int rc = nva_check_launch("linear_skinny");
-    if (rc || direct) return rc;
+    // deferred: the partial sums [real_splits][M][N] stay in scratch for a kernel that consumes them
+    if (rc || direct || defer_finish) return rc;
     const int64_t outs = M * (swiglu ? N / 2 : N);
     hipLaunchKernelGGL(linear_skinny_finish_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, stream, scratch,
                        real_splits, (const __bf16*)bias, y, y_stride, y_is_f32, swiglu, (int)M, (int)N);
+    return nva_check_launch("linear_skinny_finish");
+}
+
+// The finishing pass alone, for partial sums that were left by a call with defer_finish.
+NVA_EXPORT int nva_linear_skinny_finish_bf16(const float* partial, int splits, const void* bias, void* y,
+                                             int64_t y_stride, int y_is_f32, int swiglu, int64_t M, int64_t N,
+                                             hipStream_t stream) {
+    if (M == 0 || N == 0) return 0;
+    if (!partial || splits <= 0 || M < 0 || N < 0 || N > 0x7fffffff || M > 0x7fffffff)
+        return nva_fail("linear_skinny_finish: bad arguments");
+    const int64_t outs = M * (swiglu ? N / 2 : N);
+    hipLaunchKernelGGL(linear_skinny_finish_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, stream, partial,
+                       splits, (const __bf16*)bias, y, y_stride, y_is_f32, swiglu, (int)M, (int)N);
     return nva_check_launch("linear_skinny_finish");
 }
 

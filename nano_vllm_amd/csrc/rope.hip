@@ -6,7 +6,7 @@
 //          position (nanovllm/layers/rotary_embedding.py:6-14,44-47), in float, one rounding;
 //          q is written back in place, k in place and into its page slot;
 //   v:     copied into its page slot (nanovllm/layers/attention.py:10-30), stored transposed.
-// Cache layouts:  K [pages, kv_heads, page_size, head_dim],  V [pages, kv_heads, head_dim, page_size].
+// Cache layouts: K [pages, kv_heads, page_size, head_dim], V transposed in tiles of keys (common.h).
 // slot = page * page_size + offset; slot -1 writes nothing into the cache.
 #include "common.h"
 
@@ -37,7 +37,8 @@ NVA_EXPORT int NVA_NAME(nva_rotary_table)(const float* inv_freq, int half, int64
 
 template <typename T>
 __global__ void __launch_bounds__(256)
-qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, int num_q_heads, int num_kv_heads, int head_dim,
+qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, PartialInput part, T* q_out, int64_t q_out_stride,
+                          int num_q_heads, int num_kv_heads, int head_dim,
                           const void* __restrict__ q_weight, const void* __restrict__ k_weight, int w_is_f32,
                           float eps, const float* __restrict__ table,
                           const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
@@ -47,7 +48,11 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, int num_q_heads, int num_k
     const int head = blockIdx.y * (blockDim.x / NVA_WAVE) + threadIdx.x / NVA_WAVE;
     const int total_heads = num_q_heads + 2 * num_kv_heads;
     if (head >= total_heads) return;
-    T* row = qkv + t * row_stride + (int64_t)head * head_dim;
+    // The row comes from qkv, or (a product left as partial sums) from `part`; then q goes to q_out
+    // and k only into the cache.
+    T* row = part.sums ? nullptr : qkv + t * row_stride + (int64_t)head * head_dim;
+    const int row_width = (num_q_heads + 2 * num_kv_heads) * head_dim;
+    const int col0 = head * head_dim;
     const int64_t slot = slots ? slots[t] : -1;
     const int half = head_dim / 2;
 
@@ -55,8 +60,10 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, int num_q_heads, int num_k
         if (slot < 0 || !v_cache) return;
         const int h = head - num_q_heads - num_kv_heads;
         const int64_t page = slot / page_size, off = slot % page_size;
-        T* dst = v_cache + ((page * num_kv_heads + h) * (int64_t)head_dim) * page_size + off;
-        for (int d = lane; d < head_dim; d += NVA_WAVE) dst[(int64_t)d * page_size] = row[d];
+        T* dst = v_cache + ((page * num_kv_heads + h) * (int64_t)head_dim) * page_size;
+        const int vt = nva_v_tile(page_size);
+        for (int d = lane; d < head_dim; d += NVA_WAVE)
+            dst[nva_v_offset((int)off, d, head_dim, vt)] = part.sums ? from_float<T>(partial_value<T>(part, t, row_width, col0 + d)) : row[d];
         return;
     }
 
@@ -69,8 +76,8 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, int num_q_heads, int num_k
         const int i = lane + j * NVA_WAVE;
         x1[j] = x2[j] = 0.f;
         if (i < half) {
-            x1[j] = to_float(row[i]);
-            x2[j] = to_float(row[i + half]);
+            x1[j] = part.sums ? partial_value<T>(part, t, row_width, col0 + i) : to_float(row[i]);
+            x2[j] = part.sums ? partial_value<T>(part, t, row_width, col0 + i + half) : to_float(row[i + half]);
             ss += x1[j] * x1[j] + x2[j] * x2[j];
         }
     }
@@ -115,8 +122,14 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, int num_q_heads, int num_k
         const int i = lane + j * NVA_WAVE;
         if (i < half) {
             const T a = from_float<T>(x1[j]), b = from_float<T>(x2[j]);
-            row[i] = a;
-            row[i + half] = b;
+            if (!part.sums) {
+                row[i] = a;
+                row[i + half] = b;
+            } else if (is_q) {
+                T* qo = q_out + t * q_out_stride + col0;
+                qo[i] = a;
+                qo[i + half] = b;
+            }
             if (k_dst) {
                 k_dst[i] = a;
                 k_dst[i + half] = b;
@@ -125,17 +138,13 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, int num_q_heads, int num_k
     }
 }
 
-// qkv rows hold [q heads | k heads | v heads] of head_dim each.  q_weight / k_weight may be null
-// (no norm), table may be null (no rotation), the caches may be null (nothing is stored).
-// table_rows is the number of positions the table covers; positions are checked on the host.
-NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store)(void* qkv, int64_t row_stride, int64_t tokens, int num_q_heads,
-                                                int num_kv_heads, int head_dim, const void* q_weight,
-                                                const void* k_weight, int w_is_f32, float eps, const float* table,
-                                                const int32_t* positions, const int32_t* slots, void* k_cache,
-                                                void* v_cache, int page_size, hipStream_t stream) {
+static int launch_qk(elem_t* qkv, int64_t row_stride, PartialInput part, elem_t* q_out, int64_t q_out_stride,
+                     int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, const void* q_weight,
+                     const void* k_weight, int w_is_f32, float eps, const float* table, const int32_t* positions,
+                     const int32_t* slots, void* k_cache, void* v_cache, int page_size, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("qk_norm_rope_store: bad token count %lld", (long long)tokens);
-    if (num_q_heads < 0 || num_kv_heads <= 0 || head_dim <= 0)
+    if (num_q_heads < 0 || num_kv_heads < 0 || num_q_heads + num_kv_heads == 0 || head_dim <= 0)
         return nva_fail("qk_norm_rope_store: bad heads q=%d kv=%d head_dim=%d", num_q_heads, num_kv_heads, head_dim);
     if (head_dim % 2 || head_dim / 2 > NVA_WAVE * NVA_MAX_PER_LANE)
         return nva_fail("qk_norm_rope_store: head_dim %d must be even and at most %d", head_dim,
@@ -146,10 +155,36 @@ NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store)(void* qkv, int64_t row_stride, i
     const int total = num_q_heads + 2 * num_kv_heads;
     const int waves = 4;
     dim3 grid((unsigned)tokens, (total + waves - 1) / waves);
-    hipLaunchKernelGGL(qk_norm_rope_store_kernel<elem_t>, grid, dim3(waves * NVA_WAVE), 0, stream, (elem_t*)qkv,
-                       row_stride, num_q_heads, num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table,
+    hipLaunchKernelGGL(qk_norm_rope_store_kernel<elem_t>, grid, dim3(waves * NVA_WAVE), 0, stream, qkv, row_stride, part,
+                       q_out, q_out_stride, num_q_heads, num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table,
                        positions, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size);
     return nva_check_launch("qk_norm_rope_store");
+}
+
+// qkv rows hold [q heads | k heads | v heads] of head_dim each.  q_weight / k_weight may be null
+// (no norm), table may be null (no rotation), the caches may be null (nothing is stored).
+// Positions are checked on the host against the rows of the table.
+NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store)(void* qkv, int64_t row_stride, int64_t tokens, int num_q_heads,
+                                                int num_kv_heads, int head_dim, const void* q_weight,
+                                                const void* k_weight, int w_is_f32, float eps, const float* table,
+                                                const int32_t* positions, const int32_t* slots, void* k_cache,
+                                                void* v_cache, int page_size, hipStream_t stream) {
+    return launch_qk((elem_t*)qkv, row_stride, PartialInput{nullptr, 0, 0, nullptr}, nullptr, 0, tokens, num_q_heads,
+                     num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table, positions, slots, k_cache, v_cache,
+                     page_size, stream);
+}
+
+// The same with the packed projection given as float partial sums [splits][tokens][row width]
+// (+ bias): q is written to q_out [tokens, q heads * head_dim], k and v only into the cache.
+NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store_of_partials)(
+    const float* sums, int splits, int64_t split_stride, const void* bias, void* q_out, int64_t q_out_stride,
+    int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, const void* q_weight, const void* k_weight,
+    int w_is_f32, float eps, const float* table, const int32_t* positions, const int32_t* slots, void* k_cache,
+    void* v_cache, int page_size, hipStream_t stream) {
+    if (!sums || splits <= 0 || !q_out) return nva_fail("qk_norm_rope_store_of_partials: no partial sums or no output");
+    return launch_qk(nullptr, 0, PartialInput{sums, splits, split_stride, bias}, (elem_t*)q_out, q_out_stride, tokens,
+                     num_q_heads, num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table, positions, slots,
+                     k_cache, v_cache, page_size, stream);
 }
 
 NVA_DEFINE_LAST_ERROR(nva_rope)

@@ -7,7 +7,8 @@ many rows, where the reference uses a library as well (nanovllm/layers/linear.py
 
 Cache layouts (chosen for the attention kernels):
     K [pages, kv_heads, page_size, head_dim]
-    V [pages, kv_heads, head_dim, page_size]      (transposed: keys are contiguous)
+    V [pages, kv_heads, page_size / vt, head_dim, vt]   transposed (keys of a channel are contiguous)
+                                                        in tiles of vt = v_tile(page_size) keys
 """
 from __future__ import annotations
 
@@ -22,6 +23,16 @@ from .library import KernelError
 _SUFFIX = {torch.bfloat16: "bf16", torch.float32: "f32"}
 
 c_i32, c_i64, c_f32, c_ptr = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+
+
+def v_tile(page_size: int) -> int:
+    """Keys per tile of the V cache: 32 when the page size is a multiple of 32, else the page."""
+    return 32 if page_size % 32 == 0 else page_size
+
+
+def v_cache_shape(pages: int, kv_heads: int, head_dim: int, page_size: int):
+    vt = v_tile(page_size)
+    return (pages, kv_heads, page_size // vt, head_dim, vt)
 
 
 def _p(t: Optional[torch.Tensor]):
@@ -48,6 +59,32 @@ def _i32(t: torch.Tensor, n: int, what: str):
         raise KernelError(f"{what}: expected contiguous int32[{n}], got {t.dtype}{tuple(t.shape)}")
 
 
+class SplitSum:
+    """A bfloat16 product left as float partial sums [splits, rows, width] (+ bias) by the
+    weight-streaming kernel, for the next kernel to add up while it reads them: the norms and
+    the q/k preparation take it in place of a tensor; anything else gets `tensor()`."""
+
+    def __init__(self, kernels, sums: torch.Tensor, splits: int, rows: int, width: int, bias):
+        self.kernels, self.sums, self.splits, self.rows, self.width, self.bias = kernels, sums, splits, rows, width, bias
+        self.dtype = torch.bfloat16
+        self.device = sums.device
+        self.shape = (rows, width)
+        self._tensor = None
+
+    def tensor(self) -> torch.Tensor:
+        if self._tensor is None:
+            out = torch.empty(self.shape, dtype=self.dtype, device=self.device)
+            library.call("gemm_skinny", "bf16", "nva_linear_skinny_finish", _p(self.sums), c_i32(self.splits),
+                         _p(self.bias), _p(out), c_i64(self.width), c_i32(0), c_i32(0), c_i64(self.rows),
+                         c_i64(self.width), self.kernels._stream())
+            self._tensor = out
+        return self._tensor
+
+
+def _t(x):
+    return x.tensor() if isinstance(x, SplitSum) else x
+
+
 class HipKernels:
     """Every device operation of the engine.  Needs a GPU and the compiled libraries."""
 
@@ -66,6 +103,8 @@ class HipKernels:
         self.fault_flag = torch.zeros(1, dtype=torch.int32, device=self.device)
         # Rows up to which the bfloat16 product runs on the engine's own kernels.
         self.own_matmul_rows = 16
+        self.skinny_target_waves = 2048     # the k range of a few-row product is split until this many waves run
+        self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
         self.mfma_attention = True
 
@@ -112,7 +151,27 @@ class HipKernels:
             raise KernelError(f"norm weight is {weight.dtype}; expected float32 or the input's {x.dtype}")
         return 0
 
+    def _norm_of_partials(self, x: "SplitSum", residual, weight, eps, out):
+        rows, width = x.shape
+        wf = self._norm_weight(weight, width, x)
+        rs = 0
+        if residual is not None:
+            rrows, rw, rs = _rows2d(residual, "add_rms_norm residual")
+            if (rrows, rw) != (rows, width) or residual.dtype != x.dtype:
+                raise KernelError("add_rms_norm: residual does not match the input")
+        if out is None:
+            out = torch.empty((rows, width), dtype=x.dtype, device=x.device)
+        orows, ow, os_ = _rows2d(out, "rms_norm output")
+        if (orows, ow) != (rows, width) or out.dtype != x.dtype:
+            raise KernelError("rms_norm: output does not match the input")
+        library.call("norm", "bf16", "nva_rms_norm_of_partials", _p(x.sums), c_i32(x.splits), c_i64(rows * width),
+                     _p(x.bias), _p(residual), c_i64(rs), _p(weight), c_i32(wf), _p(out), c_i64(os_), c_i64(rows),
+                     c_i32(width), c_f32(eps), self._stream())
+        return out
+
     def rms_norm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None):
+        if isinstance(x, SplitSum):
+            return self._norm_of_partials(x, None, weight, eps, out)
         rows, width, xs = _rows2d(x, "rms_norm input")
         wf = self._norm_weight(weight, width, x)
         if out is None:
@@ -127,6 +186,8 @@ class HipKernels:
     def add_rms_norm(self, x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor, eps: float,
                      out: Optional[torch.Tensor] = None):
         """residual <- x + residual (in place); returns (norm(residual) * weight, residual)."""
+        if isinstance(x, SplitSum):
+            return self._norm_of_partials(x, residual, weight, eps, out), residual
         rows, width, xs = _rows2d(x, "add_rms_norm input")
         rrows, rw, rs = _rows2d(residual, "add_rms_norm residual")
         if (rrows, rw) != (rows, width) or residual.dtype != x.dtype:
@@ -143,6 +204,7 @@ class HipKernels:
 
     # ------------------------------------------------------------------ feed-forward
     def silu_mul(self, gate_up: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        gate_up = _t(gate_up)
         rows, width, xs = _rows2d(gate_up, "silu_mul input")
         if width % 2:
             raise KernelError("silu_mul: the input holds gate and up halves, its width must be even")
@@ -158,9 +220,12 @@ class HipKernels:
 
     # ------------------------------------------------------------------ matrix products
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-               out_float32: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+               out_float32: bool = False, out: Optional[torch.Tensor] = None, deferred: bool = False):
         """y = x @ weight.T (+ bias), weight [out, in].  float32 inputs run the engine's own
-        float kernel; bfloat16 inputs with many rows run the library product."""
+        float kernel; bfloat16 inputs with many rows run the library product, with few rows the
+        weight-streaming kernel.  deferred: the caller hands the result to a norm or to the q/k
+        preparation only, so a product split over k may come back as a SplitSum."""
+        x = _t(x)
         m, k, xs = _rows2d(x, "linear input")
         n, wk, ws = _rows2d(weight, "linear weight")
         if wk != k or weight.dtype != x.dtype:
@@ -169,6 +234,8 @@ class HipKernels:
             raise KernelError("linear: bias does not fit")
         out_dtype = torch.float32 if out_float32 else x.dtype
         if x.dtype == torch.bfloat16 and self._skinny_takes(x, xs, weight, ws, k):
+            if deferred and 0 < m <= self.own_matmul_rows and not out_float32 and out is None and self.fuse_split_sums:
+                return self._linear_skinny(x, xs, weight, ws, bias, None, 0, False, False, m, n, k, defer=True)
             if m <= self.own_matmul_rows or out_float32:
                 if out is None:
                     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
@@ -199,19 +266,30 @@ class HipKernels:
     def _skinny_takes(x, xs, weight, ws, k) -> bool:
         return k % 8 == 0 and xs % 8 == 0 and ws % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
 
-    def _linear_skinny(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k):
+    def _linear_skinny(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k, defer=False):
         """The weight-streaming kernel for at most 16 rows; k is split over workgroups when the
-        output is too narrow to fill the GPU."""
+        output is too narrow to fill the GPU.  defer: the partial sums are returned as a SplitSum
+        (or the finished tensor, where k is not split)."""
         tiles = (n + 15) // 16
-        splits = max(1, min((2048 + tiles - 1) // tiles, k // 256))
+        splits = max(1, min((self.skinny_target_waves + tiles - 1) // tiles, k // 256))
+        if defer and splits == 1:
+            defer = False
+            out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+            os_ = n
         direct = splits == 1 and bias is None and not swiglu
         scratch = None if direct else torch.empty(splits * m * n, dtype=torch.float32, device=x.device)
-        library.call("gemm_skinny", "bf16", "nva_linear_skinny", _p(x), c_i64(xs), _p(weight), c_i64(ws), _p(bias),
-                     _p(out), c_i64(os_), c_i32(1 if out_float32 else 0), c_i32(1 if swiglu else 0), _p(scratch),
-                     c_i32(splits), c_i64(m), c_i64(n), c_i64(k), self._stream())
+        used = ctypes.c_int(0)
+        library.call("gemm_skinny", "bf16", "nva_linear_skinny", _p(x), c_i64(xs), _p(weight), c_i64(ws),
+                     None if defer else _p(bias), _p(out), c_i64(os_), c_i32(1 if out_float32 else 0),
+                     c_i32(1 if swiglu else 0), _p(scratch), c_i32(splits), c_i32(1 if defer else 0), c_i64(m), c_i64(n),
+                     c_i64(k), ctypes.byref(used), self._stream())
+        if defer:
+            return SplitSum(self, scratch, used.value, m, n, bias)
+        return out
 
     def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         """silu(x @ Wg.T) * (x @ Wu.T) with weight = [Wg; Wu]."""
+        x = _t(x)
         m, k, xs = _rows2d(x, "linear input")
         n, wk, ws = _rows2d(weight, "linear weight")
         if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
@@ -239,6 +317,9 @@ class HipKernels:
                            v_cache: Optional[torch.Tensor]) -> torch.Tensor:
         """Per-head norm of q and k, rotation by the table's rows, q and k written back in
         place, k and v written into their page slots.  Returns the q view [T, heads*head_dim]."""
+        if isinstance(qkv, SplitSum):
+            return self._qk_of_partials(qkv, num_heads, num_kv_heads, head_dim, q_weight, k_weight, eps, table,
+                                        positions, slots, k_cache, v_cache)
         tokens, width, stride = _rows2d(qkv, "qkv")
         if width != (num_heads + 2 * num_kv_heads) * head_dim:
             raise KernelError(f"qkv width {width} is not (heads + 2*kv_heads) * head_dim = "
@@ -265,12 +346,40 @@ class HipKernels:
                      self._stream())
         return qkv[:, : num_heads * head_dim]
 
+    def _qk_of_partials(self, qkv: "SplitSum", num_heads, num_kv_heads, head_dim, q_weight, k_weight, eps, table,
+                        positions, slots, k_cache, v_cache) -> torch.Tensor:
+        tokens, width = qkv.shape
+        if width != (num_heads + 2 * num_kv_heads) * head_dim:
+            raise KernelError("qkv width is not (heads + 2*kv_heads) * head_dim")
+        wf = 0
+        for w in (q_weight, k_weight):
+            if w is not None:
+                wf = self._norm_weight(w, head_dim, qkv)
+        if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
+            raise KernelError("qk norm: the two weights differ in type")
+        if table is not None:
+            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != head_dim or not table.is_contiguous():
+                raise KernelError(f"rotary table must be float32 [positions, {head_dim}]")
+            _i32(positions, tokens, "positions")
+        page_size = 0
+        if k_cache is not None:
+            page_size = self._check_cache(k_cache, v_cache, num_kv_heads, head_dim, qkv.dtype)
+            _i32(slots, tokens, "slots")
+        q = torch.empty((tokens, num_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+        library.call("rope", "bf16", "nva_qk_norm_rope_store_of_partials", _p(qkv.sums), c_i32(qkv.splits),
+                     c_i64(tokens * width), _p(qkv.bias), _p(q), c_i64(num_heads * head_dim), c_i64(tokens),
+                     c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim), _p(q_weight), _p(k_weight), c_i32(wf),
+                     c_f32(eps), _p(table), _p(positions), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size),
+                     self._stream())
+        return q
+
     @staticmethod
     def _check_cache(k_cache, v_cache, num_kv_heads, head_dim, dtype) -> int:
-        if k_cache.dim() != 4 or v_cache is None or v_cache.dim() != 4:
-            raise KernelError("cache tensors must be K [pages, kv_heads, page, head_dim] and V [pages, kv_heads, head_dim, page]")
+        if k_cache.dim() != 4 or v_cache is None or v_cache.dim() != 5:
+            raise KernelError("cache tensors must be K [pages, kv_heads, page, head_dim] and "
+                              "V [pages, kv_heads, page / vt, head_dim, vt]")
         pages, h, page_size, d = k_cache.shape
-        if (h, d) != (num_kv_heads, head_dim) or tuple(v_cache.shape) != (pages, h, d, page_size):
+        if (h, d) != (num_kv_heads, head_dim) or tuple(v_cache.shape) != v_cache_shape(pages, h, d, page_size):
             raise KernelError(f"cache shapes K {tuple(k_cache.shape)} V {tuple(v_cache.shape)} do not fit "
                               f"{num_kv_heads} kv heads of {head_dim}")
         if not (k_cache.is_contiguous() and v_cache.is_contiguous()) or k_cache.dtype != dtype or v_cache.dtype != dtype:
@@ -283,6 +392,7 @@ class HipKernels:
                         window: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Causal attention of the step's tokens over the cache.  `batch` is the step's
         StepBatch; `group` selects its block tables.  q [T, heads*head_dim] (rows may be strided)."""
+        q = _t(q)
         tokens, width, qs = _rows2d(q, "attention q")
         if width != num_heads * head_dim:
             raise KernelError("attention: q width is not heads * head_dim")
@@ -344,6 +454,8 @@ class HipKernels:
             if n * num_kv_heads * ((max_kv + cand - 1) // cand) >= 2048:
                 split_len = cand
                 break
+        # a wave keeps its split's block table entries in one register per lane: at most 62 pages
+        split_len = max(32, min(split_len, (62 * page_size) // 32 * 32))
         num_splits = (max_kv + split_len - 1) // split_len
         scratch = None
         if num_splits > 1:

@@ -81,14 +81,16 @@ class Attention(Part):
         k = self.kernels
         w = self.weights
         kv_heads = 0 if self.shared else self.kv_heads
-        qkv = k.linear(x, w["qkv_proj.weight"], w.get("qkv_proj.bias"))
+        # deferred: the products below are handed to the q/k preparation and to the block's norm only
+        pe = self.position_encoding
+        table = pe.rotary_table() if pe is not None else None
+        # deferred: the products below are handed to the q/k preparation and to the block's norm only
+        qkv = k.linear(x, w["qkv_proj.weight"], w.get("qkv_proj.bias"), deferred=pe is None or table is not None)
         group = batch.groups[cache.group]
         slots = None if self.shared else group.slot_mapping
         kc, vc = (None, None) if self.shared else (cache.k, cache.v)
         qw = w.get("q_norm.weight")
         kw = w.get("k_norm.weight")
-        pe = self.position_encoding
-        table = pe.rotary_table() if pe is not None else None
         if pe is None or table is not None:
             q = k.qk_norm_rope_store(qkv, self.heads, kv_heads, self.head_dim, qw, kw, self.eps, table,
                                      batch.positions, slots, kc, vc)
@@ -104,7 +106,7 @@ class Attention(Part):
                                      slots, kc, vc)
         o = k.paged_attention(q, self.heads, self.kv_heads, self.head_dim, cache.k, cache.v, batch, cache.group,
                               self.scale, self.window)
-        return k.linear(o, w[f"{self.o_name}.weight"])
+        return k.linear(o, w[f"{self.o_name}.weight"], deferred=True)
 
 
 register_part("mixer", "attention", Attention)

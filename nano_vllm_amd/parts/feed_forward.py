@@ -33,7 +33,8 @@ class SwiGLU(Part):
 
     def forward(self, x, batch=None):
         z = self.kernels.linear_silu_mul(x, self.weights["gate_up_proj.weight"])
-        return self.kernels.linear(z, self.weights[f"{self.down_name}.weight"])
+        # deferred: the block hands this to the next norm only
+        return self.kernels.linear(z, self.weights[f"{self.down_name}.weight"], deferred=True)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

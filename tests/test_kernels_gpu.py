@@ -10,7 +10,7 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
-from torch_kernels import TorchKernels
+from torch_kernels import TorchKernels, new_caches
 
 pytestmark = pytest.mark.gpu
 
@@ -160,6 +160,44 @@ def test_linear_silu_mul(hip, ref, m, inner, k):
     _close(hip[torch.float32].linear_silu_mul(xf, wf), ref.linear_silu_mul(xf, wf), torch.float32)
 
 
+def test_split_products_are_consumed_by_norm_and_qk_kernels(hip, ref):
+    """A product left as partial sums gives, through the kernels that take it, bit for bit what the
+    finished product gives."""
+    from nano_vllm_amd.kernels.ops import SplitSum
+    k = hip[torch.bfloat16]
+    m, kk = 5, 4096
+    x = _rand((m, kk), torch.bfloat16, 30)
+    # output projection -> fused residual sum and norm
+    w = _rand((256, kk), torch.bfloat16, 31, 0.05)
+    y = k.linear(x, w, deferred=True)
+    assert isinstance(y, SplitSum) and y.splits > 1
+    done = k.linear(x, w)
+    assert torch.equal(y.tensor(), done)
+    res = _rand((m, 256), torch.bfloat16, 32)
+    nw = _rand((256,), torch.bfloat16, 33) + 1
+    r1, r2 = res.clone(), res.clone()
+    a, _ = k.add_rms_norm(y, r1, nw, 1e-6)
+    b, _ = k.add_rms_norm(done, r2, nw, 1e-6)
+    assert torch.equal(a, b) and torch.equal(r1, r2)
+    assert torch.equal(k.rms_norm(y, nw, 1e-6), k.rms_norm(done, nw, 1e-6))
+    # packed q/k/v projection with a bias -> norm, rotation and cache write
+    hq, hkv, D, page = 6, 2, 64, 16
+    wq = _rand(((hq + 2 * hkv) * D, kk), torch.bfloat16, 34, 0.05)
+    bias = _rand(((hq + 2 * hkv) * D,), torch.bfloat16, 35)
+    qkv = k.linear(x, wq, bias, deferred=True)
+    assert isinstance(qkv, SplitSum)
+    full = k.linear(x, wq, bias)
+    table = ref.rotary_table(_inv_freq(D, 1e4), 100)
+    positions = torch.tensor([3, 50, 7, 99, 0], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([17, 2, 40, -1, 33], dtype=torch.int32, device=DEV)
+    qn, kn = _rand((D,), torch.bfloat16, 36) + 1, _rand((D,), torch.bfloat16, 37) + 1
+    caches = [new_caches(4, hkv, D, page, torch.bfloat16, DEV) for _ in range(2)]
+    q1 = k.qk_norm_rope_store(qkv, hq, hkv, D, qn, kn, 1e-6, table, positions, slots, *caches[0])
+    q2 = k.qk_norm_rope_store(full, hq, hkv, D, qn, kn, 1e-6, table, positions, slots, *caches[1])
+    assert torch.equal(q1, q2) and torch.equal(caches[0][0], caches[1][0]) and torch.equal(caches[0][1], caches[1][1])
+    assert float(caches[0][1].abs().sum()) > 0
+
+
 # ------------------------------------------------------------------------------ rotation and cache write
 def _inv_freq(D, theta):
     return (1.0 / (theta ** (torch.arange(0, D, 2, dtype=torch.float) / D))).to(DEV)
@@ -188,8 +226,7 @@ def test_qk_norm_rope_store(hip, ref, dtype, hq, hkv, D, page, norm):
     positions = torch.randint(0, 500, (T,), dtype=torch.int32, device=DEV)
     slots = torch.randperm(pages * page)[:T].to(torch.int32).to(DEV)
     slots[5] = -1                                                   # this token is not stored
-    caches = [[torch.zeros((pages, hkv, page, D), dtype=dtype, device=DEV),
-               torch.zeros((pages, hkv, D, page), dtype=dtype, device=DEV)] for _ in range(2)]
+    caches = [new_caches(pages, hkv, D, page, dtype, DEV) for _ in range(2)]
     a, b = qkv.clone(), qkv.clone()
     qa = k.qk_norm_rope_store(a, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[0])
     qb = ref.qk_norm_rope_store(b, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[1])
@@ -223,10 +260,8 @@ def _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed, boost=None):
     total = sum(pages_per) + 3
     order = list(range(total))
     rng.shuffle(order)
-    kc = torch.zeros((total, hkv, page, D), dtype=dtype, device=DEV)
-    vc = torch.zeros((total, hkv, D, page), dtype=dtype, device=DEV)
-    kc.normal_(0, 1.0)                                              # what unused slots hold must not matter
-    vc.normal_(0, 1.0)
+    kc, vc = new_caches(total, hkv, D, page, dtype, DEV, fill=1.0)  # what unused slots hold must not matter
+    vt = vc.shape[4]
     width = max(pages_per)
     tables = torch.full((S, width), -1, dtype=torch.int32)
     ks, vs, qs, token_seq, positions = [], [], [], [], []
@@ -243,7 +278,7 @@ def _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed, boost=None):
             q[:, :, 0] = 8.0
         for j in range(n):
             kc[mine[j // page], :, j % page, :] = k[j]
-            vc[mine[j // page], :, :, j % page] = v[j]
+            vc[mine[j // page], :, (j % page) // vt, :, (j % page) % vt] = v[j]
         ks.append(k); vs.append(v); qs.append(q)
         token_seq += [s] * q_lens[s]
         positions += list(range(n - q_lens[s], n))

@@ -95,8 +95,9 @@ def _attention_setup(dtype, window=None, qk_norm=True, heads=6, kv_heads=3, D=32
         part.weights["k_norm.weight"] = w["k_norm.weight"].to(DEV)
     need = part.cache_need()
     cache = CacheManager([CacheGroup(window, (0,))], page, pages, enable_prefix_caching=False)
-    lc = LayerCache(group=0, k=torch.zeros((pages, need.num_kv_heads, page, need.head_dim), dtype=dtype, device=DEV),
-                    v=torch.zeros((pages, need.num_kv_heads, need.head_dim, page), dtype=dtype, device=DEV))
+    from torch_kernels import new_caches
+    kc, vc = new_caches(pages, need.num_kv_heads, need.head_dim, page, dtype, DEV)
+    lc = LayerCache(group=0, k=kc, v=vc)
     pcfg = plain.PlainConfig(vocab_size=10, hidden_size=hidden, num_layers=1, num_heads=heads, num_kv_heads=kv_heads,
                              head_dim=D, intermediate_size=1, rms_norm_eps=1e-6, rope_theta=1e4, max_position=256,
                              tie_word_embeddings=False, attention_bias=False)

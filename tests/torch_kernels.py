@@ -14,6 +14,22 @@ def _round(x, dtype):
     return x.to(dtype).to(torch.float32)
 
 
+def v_tile(page_size: int) -> int:
+    """Keys per tile of the V cache [pages, kv_heads, page / vt, head_dim, vt]."""
+    return 32 if page_size % 32 == 0 else page_size
+
+
+def new_caches(pages, kv_heads, head_dim, page_size, dtype, device, fill=None):
+    """K [pages, kv_heads, page, head_dim] and V [pages, kv_heads, page / vt, head_dim, vt]."""
+    vt = v_tile(page_size)
+    k = torch.zeros((pages, kv_heads, page_size, head_dim), dtype=dtype, device=device)
+    v = torch.zeros((pages, kv_heads, page_size // vt, head_dim, vt), dtype=dtype, device=device)
+    if fill is not None:
+        k.normal_(0, fill)
+        v.normal_(0, fill)
+    return k, v
+
+
 class TorchKernels:
     name = "torch-plain"
 
@@ -65,7 +81,7 @@ class TorchKernels:
             return out
         return y
 
-    def linear(self, x, weight, bias=None, out_float32=False, out=None):
+    def linear(self, x, weight, bias=None, out_float32=False, out=None, deferred=False):
         y = x.float() @ weight.float().T
         if bias is not None:
             y = y + bias.float()
@@ -114,8 +130,9 @@ class TorchKernels:
                 s = slots.long()
                 ok = s >= 0
                 page, off = s[ok] // page_size, s[ok] % page_size
+                vt = v_cache.shape[4]
                 k_cache[page, :, off, :] = k[ok]
-                v_cache[page, :, :, off] = v[ok]
+                v_cache[page, :, off // vt, :, off % vt] = v[ok]
         return qkv[:, :qd]
 
     # attention (attention.py:64-75): token by token through the block table
@@ -135,7 +152,8 @@ class TorchKernels:
             assert bool((pages >= 0).all()), "a visible key has no page"
             offs = js % page_size
             keys = k_cache[pages, :, offs, :].float()                # [n, Hkv, D]
-            vals = v_cache[pages, :, :, offs].float()                # [n, Hkv, D]
+            vt = v_cache.shape[4]
+            vals = v_cache[pages, :, offs // vt, :, offs % vt].float()   # [n, Hkv, D]
             qt = q[t].float().reshape(num_heads, D)
             for h in range(num_heads):
                 s = (keys[:, h // G] @ qt[h]) * scale
