@@ -49,8 +49,7 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
 
     const int n0 = (blockIdx.x * SK_WAVES + wave) * 16;
     const bool active = n0 < N;                       // idle waves still help to stage x
-    const int wrow = min(n0 + col, N - 1);
-    const __bf16* wp = w + (int64_t)wrow * w_stride + 32 * g;
+    const __bf16* wrow = w + (int64_t)min(n0 + col, N - 1) * w_stride;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 
     for (int c_begin = k_begin; c_begin < k_end; c_begin += chunk) {
@@ -68,14 +67,17 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
         if (!active) continue;
         const __bf16* xp = x_s + col * xs_stride + 32 * g - c_begin;
 
+        // Every load of W is unconditional (an offset past the chunk is moved back into the row: what
+        // it reads meets zeros of x_s or is dropped), and the loads of the next step are issued before
+        // the products of the current one on a single path through the loop, so that the wait before
+        // the products covers the current step's loads only.
+        const int k_last = K - 8;
         bf16x8 a_next[SK_UNROLL][4];
 #pragma unroll
         for (int u = 0; u < SK_UNROLL; ++u)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int k = c_begin + u * SK_KSTEP + 32 * g + 8 * c;
-                a_next[u][c] = k < c_end ? *reinterpret_cast<const bf16x8*>(wp + c_begin + u * SK_KSTEP + 8 * c) : zero8();
-            }
+            for (int c = 0; c < 4; ++c)
+                a_next[u][c] = *reinterpret_cast<const bf16x8*>(wrow + min(c_begin + u * SK_KSTEP + 32 * g + 8 * c, k_last));
         for (int kk = c_begin; kk < c_end; kk += SK_KSTEP * SK_UNROLL) {
             bf16x8 a[SK_UNROLL][4];
 #pragma unroll
@@ -83,24 +85,19 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
 #pragma unroll
                 for (int c = 0; c < 4; ++c) a[u][c] = a_next[u][c];
             const int kn = kk + SK_KSTEP * SK_UNROLL;
-            if (kn < c_end) {
 #pragma unroll
-                for (int u = 0; u < SK_UNROLL; ++u)
+            for (int u = 0; u < SK_UNROLL; ++u)
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        const int k = kn + u * SK_KSTEP + 32 * g + 8 * c;
-                        a_next[u][c] = k < c_end ? *reinterpret_cast<const bf16x8*>(wp + kn + u * SK_KSTEP + 8 * c) : zero8();
-                    }
-            }
+                for (int c = 0; c < 4; ++c)
+                    a_next[u][c] = *reinterpret_cast<const bf16x8*>(wrow + min(kn + u * SK_KSTEP + 32 * g + 8 * c, k_last));
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u) {
-                if (kk + u * SK_KSTEP < c_end) {
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        // x_s holds zeros beyond c_end, up to the padded end of the chunk
-                        const bf16x8 b = *reinterpret_cast<const bf16x8*>(xp + kk + u * SK_KSTEP + 8 * c);
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][c], b, acc, 0, 0, 0);
-                    }
+                for (int c = 0; c < 4; ++c) {
+                    // x_s holds zeros from c_end to the padded end of the chunk
+                    const bf16x8 b = *reinterpret_cast<const bf16x8*>(xp + min(kk + u * SK_KSTEP, c_begin + chunk - SK_KSTEP) + 8 * c);
+                    const bool live = kk + u * SK_KSTEP < c_begin + chunk;
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][c], live ? b : zero8(), acc, 0, 0, 0);
                 }
             }
         }
