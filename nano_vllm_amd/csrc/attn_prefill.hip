@@ -29,7 +29,8 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 #define PF_WAVES 4
 
 template <int D>
-__global__ void __launch_bounds__(PF_WAVES * NVA_WAVE)
+// two waves per SIMD (at most 256 registers) up to head_dim 128; beyond that the accumulators need more
+__global__ void __launch_bounds__(PF_WAVES * NVA_WAVE, D <= 128 ? 2 : 1)
 attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
                     const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                     const int32_t* __restrict__ block_tables, int table_stride,
@@ -104,51 +105,76 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     const int a_r = col >> 3, h_r = (col >> 2) & 1, b_r = col & 3;
     const int row_key = 16 * (a_r >> 1) + 8 * h_r + 4 * (a_r & 1) + b_r;
     const int first_row = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+    const float c_exp = scale * 1.4426950408889634f;      // scale * log2(e)
+
+    // ---- the request's block table entries for the keys this workgroup reads, once, into LDS
+    extern __shared__ int32_t table_s[];
+    const int page_lo = kb_lo / page_size;
+    const int num_pages = (kb_hi - 1) / page_size - page_lo + 1;
+    for (int i = tid; i < num_pages; i += PF_WAVES * NVA_WAVE) {
+        const int page = table[page_lo + i];
+        if (page < 0 && error_flag) atomicOr(error_flag, 2);
+        table_s[i] = max(page, 0);
+    }
+    __syncthreads();
+
+    // Staging of a tile, per thread: PIECES 16-byte pieces of K (row r = tid / (D/8) + i * 256 / (D/8))
+    // and of V (channel d = tid / 8 + 32 i, the 8 keys of group tid % 8).  Every load is unconditional:
+    // a key outside the visible range is replaced by the nearest visible one (its scores are masked by
+    // the key index; V is zeroed when it is written to LDS, in the tiles at the two ends only).  The
+    // loads of tile t + 1 are issued before the products of tile t.
+    constexpr int PIECES = PF_BN * (D / 8) / (PF_WAVES * NVA_WAVE);
+    static_assert(PF_BN * (D / 8) % (PF_WAVES * NVA_WAVE) == 0, "the tile divides over the threads");
+    const int last_key = kb_hi - 1;
+    bf16x8 k_reg[PIECES], v_reg[PIECES];
+    auto issue_loads = [&](int kb) {
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int idx = tid + i * PF_WAVES * NVA_WAVE;
+            const int r = idx / (D / 8), piece = idx % (D / 8);
+            const int key = min(max(kb + r, first_any), last_key);
+            const int page = table_s[key / page_size - page_lo];
+            k_reg[i] = *reinterpret_cast<const bf16x8*>(
+                k_cache + (((int64_t)page * num_kv_heads + kvh) * page_size + key % page_size) * D + piece * 8);
+        }
+        const int grp = tid % (PF_BN / 8);
+        const int key0 = min(max(kb + grp * 8, first_any & ~7), last_key & ~7);
+        const int page = table_s[key0 / page_size - page_lo];
+        const __bf16* vb = v_cache + ((int64_t)page * num_kv_heads + kvh) * D * (int64_t)page_size;
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int d = tid / (PF_BN / 8) + i * (PF_WAVES * NVA_WAVE / (PF_BN / 8));
+            v_reg[i] = *reinterpret_cast<const bf16x8*>(vb + nva_v_offset(key0 % page_size, d, D, vt));
+        }
+    };
+    issue_loads(kb_lo);
 
     for (int kb = kb_lo; kb < kb_hi; kb += PF_BN) {
-        // ---- stage the K tile: 64 rows of D channels
-        for (int idx = tid; idx < PF_BN * (D / 8); idx += PF_WAVES * NVA_WAVE) {
+        // ---- registers -> LDS
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) {
+            const int idx = tid + i * PF_WAVES * NVA_WAVE;
             const int r = idx / (D / 8), piece = idx % (D / 8);
-            const int key = kb + r;
-            bf16x8 v;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
-            if (key >= first_any && key < kb_hi) {
-                const int page = table[key / page_size];
-                if (page < 0) {
-                    if (error_flag) atomicOr(error_flag, 2);
-                } else {
-                    v = *reinterpret_cast<const bf16x8*>(
-                        k_cache + (((int64_t)page * num_kv_heads + kvh) * page_size + key % page_size) * D + piece * 8);
-                }
-            }
-            *reinterpret_cast<bf16x8*>(&k_s[r * KS + piece * 8]) = v;
+            *reinterpret_cast<bf16x8*>(&k_s[r * KS + piece * 8]) = k_reg[i];
         }
-        // ---- stage the V tile: D rows of 64 keys (8 keys = 16 bytes lie in one page)
-        for (int idx = tid; idx < D * (PF_BN / 8); idx += PF_WAVES * NVA_WAVE) {
-            const int d = idx / (PF_BN / 8), grp = idx % (PF_BN / 8);
+        {
+            const int grp = tid % (PF_BN / 8);
             const int key0 = kb + grp * 8;
-            bf16x8 v;
+            const bool edge = kb < first_any || kb + PF_BN > kb_hi;          // the same for the whole workgroup
 #pragma unroll
-            for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
-            if (key0 + 8 > first_any && key0 < kb_hi) {
-                const int page = table[key0 / page_size];
-                if (page < 0) {
-                    if (error_flag) atomicOr(error_flag, 2);
-                } else {
-                    v = *reinterpret_cast<const bf16x8*>(
-                        v_cache + ((int64_t)page * num_kv_heads + kvh) * D * (int64_t)page_size +
-                        nva_v_offset(key0 % page_size, d, D, vt));
-                    if (key0 + 8 > kb_hi || key0 < first_any) {
+            for (int i = 0; i < PIECES; ++i) {
+                const int d = tid / (PF_BN / 8) + i * (PF_WAVES * NVA_WAVE / (PF_BN / 8));
+                bf16x8 v = v_reg[i];
+                if (edge) {
 #pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (key0 + e >= kb_hi || key0 + e < first_any) v[e] = (__bf16)0.f;
-                    }
+                    for (int e = 0; e < 8; ++e)
+                        if (key0 + e >= kb_hi || key0 + e < first_any) v[e] = (__bf16)0.f;
                 }
+                *reinterpret_cast<bf16x8*>(&v_s[d * VS + grp * 8]) = v;
             }
-            *reinterpret_cast<bf16x8*>(&v_s[d * VS + grp * 8]) = v;
         }
         __syncthreads();
+        issue_loads(min(kb + PF_BN, last_key & ~(PF_BN - 1)));               // after the last tile: read again, dropped
 
         if (active) {
             // ---- scores of 2 x 32 keys
@@ -164,43 +190,54 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                     s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[c], s[kt], 0, 0, 0);
                 }
             }
-            // this lane: query `col`; register e of tile kt is key kb + 32*kt + 16*(e/8) + 8*h + e%8
+            // this lane: query `col`; register e of tile kt is key kb + 32*kt + 16*(e/8) + 8*h + e%8.
+            // The maximum is taken of the raw scores (scale > 0) and the scale folded, with log2(e),
+            // into the exponent: p = 2^((s - m) * scale * log2 e), one fused multiply-add per score.
             const bool full = kb + PF_BN - 1 <= start + q0 && kb >= first_any + (window > 0 ? PF_BM : 0);
             float m_new = m_run;
+            if (!full) {
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) {
+                        const int key = kb + 32 * kt + 16 * (e >> 3) + 8 * h + (e & 7);
+                        if (key > pos || key < first_row) s[kt][e] = -INFINITY;
+                    }
+            }
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    float v = s[kt][e] * scale;
-                    if (!full) {
-                        const int key = kb + 32 * kt + 16 * (e >> 3) + 8 * h + (e & 7);
-                        if (key > pos || key < first_row) v = -INFINITY;
-                    }
-                    s[kt][e] = v;
-                    m_new = fmaxf(m_new, v);
-                }
+                for (int e = 0; e < 16; ++e) m_new = fmaxf(m_new, s[kt][e]);
             m_new = fmaxf(m_new, __shfl_xor(m_new, 32, NVA_WAVE));
+            // a row that has seen no key yet keeps -inf as its maximum; exponents then use a finite
+            // stand-in so that -inf - (-inf) never arises
+            const float m_use = fmaxf(m_new, -1e30f);
+            const float neg_mc = -m_use * c_exp;
             float psum = 0.f;
             bf16x8 pf[2][2];
 #pragma unroll
             for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const float p = (s[kt][e] == -INFINITY) ? 0.f : __expf(s[kt][e] - m_new);
-                    const __bf16 pb = (__bf16)p;
-                    pf[kt][e >> 3][e & 7] = pb;
-                    psum += (float)pb;
+                    const float p = __builtin_amdgcn_exp2f(fmaf(s[kt][e], c_exp, neg_mc));
+                    pf[kt][e >> 3][e & 7] = (__bf16)p;
+                    psum += p;
                 }
             psum += __shfl_xor(psum, 32, NVA_WAVE);
-            const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
+            // The accumulators are rescaled only when some row of the wave has a new maximum (after the
+            // first tiles of a row that is rare): alpha is exactly 1 otherwise.
+            const float alpha = __builtin_amdgcn_exp2f((fmaxf(m_run, -1e30f) - m_use) * c_exp);
+            const bool rescale = __any(m_new > m_run);
             l_run = l_run * alpha + psum;
             m_run = m_new;
             // ---- O^T += V^T P^T
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 f32x16 o = acc[mt];
+                if (rescale) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) o[e] *= alpha;
+                    for (int e = 0; e < 16; ++e) o[e] *= alpha;
+                }
                 const __bf16* vrow = &v_s[(mt * 32 + col) * VS + 8 * h];
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt)
@@ -250,9 +287,14 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
     const int64_t grid_y = (int64_t)num_kv_heads * ((G + PF_WAVES - 1) / PF_WAVES);
     if (total_tiles < 0 || total_tiles > 0x7fffffff || grid_y > 65535 || window < 0 || table_stride <= 0)
         return nva_fail("attn_prefill: bad sizes (tiles %lld, heads %lld)", (long long)total_tiles, (long long)grid_y);
+    if (table_stride > 4096) {
+        nva_fail("attn_prefill: block tables of %d pages do not fit the kernel's staging buffer", table_stride);
+        return 1;
+    }
+    const size_t table_bytes = (size_t)table_stride * sizeof(int32_t);
     dim3 grid((unsigned)total_tiles, (unsigned)grid_y);
 #define LAUNCH(DD)                                                                                                 \
-    hipLaunchKernelGGL(attn_prefill_kernel<DD>, grid, dim3(PF_WAVES * NVA_WAVE), 0, stream, (const __bf16*)q,        \
+    hipLaunchKernelGGL(attn_prefill_kernel<DD>, grid, dim3(PF_WAVES * NVA_WAVE), table_bytes, stream, (const __bf16*)q, \
                        q_stride, (__bf16*)out, out_stride, (const __bf16*)k_cache, (const __bf16*)v_cache,           \
                        block_tables, table_stride, cu_seqlens_q, kv_lens, first_seq, num_seqs, num_q_heads,          \
                        num_kv_heads, page_size, scale, window, error_flag)
