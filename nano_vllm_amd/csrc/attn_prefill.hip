@@ -113,7 +113,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     const int num_pages = (kb_hi - 1) / page_size - page_lo + 1;
     for (int i = tid; i < num_pages; i += PF_WAVES * NVA_WAVE) {
         const int page = table[page_lo + i];
-        if (page < 0 && error_flag) atomicOr(error_flag, 2);
+        // pages before the first visible key may have been given back (a window): no fault
+        if (page < 0 && page_lo + i >= first_any / page_size && error_flag) atomicOr(error_flag, 2);
         table_s[i] = max(page, 0);
     }
     __syncthreads();
