@@ -328,9 +328,9 @@ class HipKernels:
         for w in (q_weight, k_weight):
             if w is not None:
                 wf = self._norm_weight(w, head_dim, qkv)
-        if (q_weight is None) != (k_weight is None):
+        if num_kv_heads and (q_weight is None) != (k_weight is None):
             raise KernelError("qk norm: give both weights or none")
-        if q_weight is not None and q_weight.dtype != k_weight.dtype:
+        if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
             raise KernelError("qk norm: the two weights differ in type")
         if table is not None:
             if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != head_dim or not table.is_contiguous():
@@ -355,6 +355,8 @@ class HipKernels:
         for w in (q_weight, k_weight):
             if w is not None:
                 wf = self._norm_weight(w, head_dim, qkv)
+        if num_kv_heads and (q_weight is None) != (k_weight is None):
+            raise KernelError("qk norm: give both weights or none")
         if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
             raise KernelError("qk norm: the two weights differ in type")
         if table is not None:

@@ -170,3 +170,43 @@ def plain_logits(folder: str, tokens: Sequence[int], rounding=None) -> torch.Ten
 
 def rel_err(got: torch.Tensor, want: torch.Tensor) -> float:
     return float((got.double() - want.double()).abs().max() / want.double().abs().max())
+
+
+def run_mixed_groups(runner: ModelRunner, requests: Dict[str, List[int]], seed: int, max_live: int = 4):
+    """As run_mixed for models with several cache groups: a request is admitted when every
+    group can take its first portion, and a portion that finds no pages waits for a step."""
+    rng = random.Random(seed)
+    waiting = list(requests)
+    live: Dict[str, int] = {}
+    got: Dict[str, List[torch.Tensor]] = {r: [] for r in requests}
+    for _ in range(100000):
+        if not waiting and not live:
+            break
+        while waiting and len(live) < max_live:
+            rid = waiting.pop(0)
+            runner.cache.admit(rid)
+            live[rid] = 0
+        entries = []
+        for rid, pos in live.items():
+            left = len(requests[rid]) - pos
+            n = 1 if left <= 20 else min(left - 20, rng.choice([2, 3, 5, 8, 13, 21]))
+            if not runner.cache.can_reserve(rid, pos + n, first_query=pos):
+                n = 1
+                if not runner.cache.can_reserve(rid, pos + 1, first_query=pos):
+                    continue
+            runner.cache.reserve(rid, pos + n, first_query=pos)
+            entries.append(StepEntry(rid, requests[rid][pos:pos + n], pos, list(range(n))))
+        assert entries, "no request can go on: the pools are too small"
+        rng.shuffle(entries)
+        logits = runner.step(entries).float().cpu()
+        row = 0
+        for e in entries:
+            n = len(e.tokens)
+            got[e.request].append(logits[row:row + n])
+            row += n
+            live[e.request] += n
+            if live[e.request] == len(requests[e.request]):
+                runner.cache.release(e.request)
+                del live[e.request]
+        runner.cache.check()
+    return {r: torch.cat(v) for r, v in got.items()}

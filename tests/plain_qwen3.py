@@ -157,9 +157,11 @@ def feed_forward(x, w_gate, w_up, w_down, rounding=None):
     return rd(silu_mul(g, u, rounding) @ w_down.T)
 
 
-def self_attention(x, positions, w, prefix, cfg: PlainConfig, window=None, rounding=None):
+def self_attention(x, positions, w, prefix, cfg: PlainConfig, window=None, rounding=None, kv=None, keep=None):
     """qwen3.py:72-88: projections, per-head q/k norm (only without bias), rotation,
-    attention, output projection."""
+    attention, output projection.  For the tests of layer orders (not a reference feature):
+    kv = (k, v) of another layer replaces this layer's own keys and values; keep, a list,
+    receives this layer's (k, v)."""
     rd = _rounder(rounding)
     T = x.shape[0]
     D = cfg.head_dim
@@ -171,33 +173,45 @@ def self_attention(x, positions, w, prefix, cfg: PlainConfig, window=None, round
         return rd(y)
 
     q = proj("q_proj").view(T, cfg.num_heads, D)
-    k = proj("k_proj").view(T, cfg.num_kv_heads, D)
-    v = proj("v_proj").view(T, cfg.num_kv_heads, D)
     if not cfg.attention_bias:                                     # qwen3.py:68-70,82-84
         q = rms_norm(q, w[f"{prefix}.q_norm.weight"], cfg.rms_norm_eps, rounding)
-        k = rms_norm(k, w[f"{prefix}.k_norm.weight"], cfg.rms_norm_eps, rounding)
     angles = rope_angles(D, positions, cfg.rope_theta)
     q = apply_rope(q, angles, rounding)
-    k = apply_rope(k, angles, rounding)
+    if kv is None:
+        k = proj("k_proj").view(T, cfg.num_kv_heads, D)
+        v = proj("v_proj").view(T, cfg.num_kv_heads, D)
+        if not cfg.attention_bias:
+            k = rms_norm(k, w[f"{prefix}.k_norm.weight"], cfg.rms_norm_eps, rounding)
+        k = apply_rope(k, angles, rounding)
+    else:
+        k, v = kv
+    if keep is not None:
+        keep.append((k, v))
     o = causal_attention(q, k, v, D ** -0.5, window, rounding)     # qwen3.py:39
     return rd(o.reshape(T, cfg.num_heads * D) @ w[f"{prefix}.o_proj.weight"].T)
 
 
-def hidden_states(w, cfg: PlainConfig, token_ids, rounding=None, first_position=0):
+def hidden_states(w, cfg: PlainConfig, token_ids, rounding=None, first_position=0, order=None, windows=None):
     """qwen3.py:173-183 with the layer of qwen3.py:146-159.  Returns the normalised
-    last hidden state of every position, [T, H]."""
+    last hidden state of every position, [T, H].  For the tests of layer orders and windows
+    (not reference features): order = [(layer, index of the earlier entry whose keys and
+    values it reads, or None)], windows = {layer: keys}."""
     ids = torch.as_tensor(token_ids, dtype=torch.long)
     positions = torch.arange(first_position, first_position + len(ids))
     h = w["model.embed_tokens.weight"][ids]                        # embed_head.py:38
     residual = None
-    for i in range(cfg.num_layers):
+    order = order if order is not None else [(i, None) for i in range(cfg.num_layers)]
+    windows = windows or {}
+    kept = []
+    for i, source in order:
         p = f"model.layers.{i}"
         if residual is None:                                       # qwen3.py:152-153
             h, residual = rms_norm(h, w[f"{p}.input_layernorm.weight"], cfg.rms_norm_eps, rounding), h
         else:                                                      # qwen3.py:154-155
             h, residual = add_rms_norm(h, residual, w[f"{p}.input_layernorm.weight"],
                                        cfg.rms_norm_eps, rounding)
-        h = self_attention(h, positions, w, f"{p}.self_attn", cfg, None, rounding)
+        h = self_attention(h, positions, w, f"{p}.self_attn", cfg, windows.get(i), rounding,
+                           kv=None if source is None else kept[source], keep=kept)
         h, residual = add_rms_norm(h, residual, w[f"{p}.post_attention_layernorm.weight"],
                                    cfg.rms_norm_eps, rounding)    # qwen3.py:157
         h = feed_forward(h, w[f"{p}.mlp.gate_proj.weight"], w[f"{p}.mlp.up_proj.weight"],
@@ -206,10 +220,10 @@ def hidden_states(w, cfg: PlainConfig, token_ids, rounding=None, first_position=
     return h
 
 
-def logits(w, cfg: PlainConfig, token_ids, rounding=None, first_position=0):
+def logits(w, cfg: PlainConfig, token_ids, rounding=None, first_position=0, order=None, windows=None):
     """Logits of every position [T, V] (embed_head.py:61; tied head: qwen3.py:202-203).
     The product with the head is left unrounded: logits are wanted in float32."""
-    h = hidden_states(w, cfg, token_ids, rounding, first_position)
+    h = hidden_states(w, cfg, token_ids, rounding, first_position, order, windows)
     head = w["model.embed_tokens.weight"] if cfg.tie_word_embeddings else w["lm_head.weight"]
     return h @ head.T
 
