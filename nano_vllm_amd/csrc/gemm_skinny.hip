@@ -1,13 +1,14 @@
-// y[M, N] = x[M, K] W[N, K]^T for few rows (M <= 16, bfloat16): the linear layers of a decode
+// y[M, N] = x[M, K] W[N, K]^T for few rows (M <= 64, bfloat16): the linear layers of a decode
 // step (nanovllm/layers/linear.py:51,73,153; embed_head.py:61), where every weight is read once
 // and the time is the time to stream W from HBM.
 //
 // One wave owns 16 output columns (16 rows of W) over a range of k.  W rows are the A operand of
-// a 16x16x32 MFMA, the rows of x its 16 columns (rows >= M idle).  A lane reads 64 contiguous bytes of its W row per step of 128 k
-// (the k index is permuted alike in both operands), straight from global into registers; the
-// workgroup's slice of x is staged in LDS.  For small N the k range is split over workgroups, each
-// writing float partial sums; a second kernel adds the partials in a fixed order, applies the
-// optional bias and the optional SwiGLU gating (W = [gate rows; up rows]) and rounds once.
+// a 16x16x32 MFMA, 16 rows of x its 16 columns (rows >= M idle); with more than 16 rows of x the
+// same W fragment feeds one MFMA per block of 16 rows.  A lane reads four 16-byte pieces of its W
+// row per step of 128 k (the k index is permuted alike in both operands), straight from global into
+// registers; the workgroup's slice of x is staged in LDS.  For small N the k range is split over
+// workgroups, each writing float partial sums; a second kernel adds the partials in a fixed order,
+// applies the optional bias and the optional SwiGLU gating (W = [gate rows; up rows]) and rounds once.
 //
 // Requires K % 8 == 0 and 16-byte aligned rows; the launcher refuses anything else and the caller
 // uses the library product or the tiled kernel.
@@ -17,10 +18,17 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-#define SK_WAVES 4
 #define SK_KSTEP 128
 #define SK_UNROLL 2
-#define SK_CHUNK 1536     // k of x staged at a time: 16 rows * (1536 + 8) * 2 bytes of LDS
+#define SK_MAX_ROWS 64
+
+// Row blocks of x (MB), waves per workgroup and the k of x staged at a time: the LDS slice is
+// 16 * MB rows * (chunk + 8) * 2 bytes.  More rows of x take more waves per workgroup, so that a
+// staged slice of x serves more rows of W, and a shorter chunk, so that two workgroups fit a CU.
+template <int MB> struct SkShape;
+template <> struct SkShape<1> { static constexpr int waves = 4, chunk = 1536; };
+template <> struct SkShape<2> { static constexpr int waves = 8, chunk = 1024; };
+template <> struct SkShape<4> { static constexpr int waves = 8, chunk = 512; };
 
 __device__ __forceinline__ bf16x8 zero8() {
     bf16x8 z;
@@ -31,32 +39,43 @@ __device__ __forceinline__ bf16x8 zero8() {
 
 // direct: 1 = the only split writes y itself (as bfloat16 or float); 0 = float partials [split][M][N]
 //
-// The workgroup's four waves share one range of k, so its slice of x (16 rows, rows >= M zero) is
-// staged once in LDS (row stride padded by 16 bytes against bank conflicts).  The loads of the next
-// step's W fragments are issued before the products of the current one.
-__global__ void __launch_bounds__(SK_WAVES * NVA_WAVE)
+// The workgroup's waves share one range of k, so its slice of x (16 * MB rows, rows >= M zero) is
+// staged once in LDS (row stride padded by 16 bytes against bank conflicts).
+template <int MB>
+__global__ void __launch_bounds__(SkShape<MB>::waves * NVA_WAVE)
 linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf16* __restrict__ w, int64_t w_stride,
                      float* __restrict__ partial, void* __restrict__ y, int64_t y_stride, int y_is_f32, int direct,
                      int M, int N, int K, int k_per_split) {
-    extern __shared__ __attribute__((aligned(16))) __bf16 x_s[];     // [16][chunk + 8]
+    constexpr int WAVES = SkShape<MB>::waves;
+    constexpr int ROWS = 16 * MB;
+    extern __shared__ __attribute__((aligned(16))) __bf16 x_s[];     // [ROWS][chunk + 8]
     const int wave = threadIdx.x / NVA_WAVE, lane = threadIdx.x % NVA_WAVE;
     const int col = lane & 15, g = lane >> 4;
     const int split = blockIdx.y;
     const int k_begin = split * k_per_split;
     const int k_end = min(K, k_begin + k_per_split);
-    const int chunk = min(k_per_split, SK_CHUNK);
+    const int chunk = min(k_per_split, SkShape<MB>::chunk);
     const int xs_stride = chunk + 8;
 
-    const int n0 = (blockIdx.x * SK_WAVES + wave) * 16;
+    const int n0 = (blockIdx.x * WAVES + wave) * 16;
     const bool active = n0 < N;                       // idle waves still help to stage x
     const __bf16* wrow = w + (int64_t)min(n0 + col, N - 1) * w_stride;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+    // Lane (row, g) takes the 16-byte piece g + 4c of its row's 256 bytes in load c, so that one load
+    // instruction covers 64 contiguous bytes of each of the wave's 16 rows; x is read from LDS at the
+    // same k.  Every load of W is unconditional (an offset past the end of the row is moved back into
+    // it: what it reads meets zeros of x_s or is dropped).  The loads of a step are issued at its top
+    // and the products wait for them one by one; other waves of the CU cover the latency.  (Loads
+    // issued a step ahead were measured slower, and they read past the split's range of k.)
+    const int k_last = K - 8;
     for (int c_begin = k_begin; c_begin < k_end; c_begin += chunk) {
         const int c_end = min(k_end, c_begin + chunk);
-        // ---- stage x[0:16][c_begin:c_begin + chunk] (zeros beyond M and c_end)
+        // ---- stage x[0:ROWS][c_begin:c_begin + chunk] (zeros beyond M and c_end)
         __syncthreads();
-        for (int idx = threadIdx.x; idx < 16 * (chunk / 8); idx += SK_WAVES * NVA_WAVE) {
+        for (int idx = threadIdx.x; idx < ROWS * (chunk / 8); idx += WAVES * NVA_WAVE) {
             const int m = idx / (chunk / 8), piece = idx % (chunk / 8);
             const int k = c_begin + piece * 8;
             bf16x8 v = zero8();
@@ -65,67 +84,58 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
         }
         __syncthreads();
         if (!active) continue;
-        const __bf16* xp = x_s + col * xs_stride + 32 * g - c_begin;
+        const __bf16* xp = x_s + col * xs_stride + 8 * g - c_begin;
 
-        // Every load of W is unconditional (an offset past the chunk is moved back into the row: what
-        // it reads meets zeros of x_s or is dropped), and the loads of the next step are issued before
-        // the products of the current one on a single path through the loop, so that the wait before
-        // the products covers the current step's loads only.
-        const int k_last = K - 8;
-        bf16x8 a_next[SK_UNROLL][4];
-#pragma unroll
-        for (int u = 0; u < SK_UNROLL; ++u)
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                a_next[u][c] = *reinterpret_cast<const bf16x8*>(wrow + min(c_begin + u * SK_KSTEP + 32 * g + 8 * c, k_last));
         for (int kk = c_begin; kk < c_end; kk += SK_KSTEP * SK_UNROLL) {
             bf16x8 a[SK_UNROLL][4];
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u)
 #pragma unroll
-                for (int c = 0; c < 4; ++c) a[u][c] = a_next[u][c];
-            const int kn = kk + SK_KSTEP * SK_UNROLL;
-#pragma unroll
-            for (int u = 0; u < SK_UNROLL; ++u)
-#pragma unroll
                 for (int c = 0; c < 4; ++c)
-                    a_next[u][c] = *reinterpret_cast<const bf16x8*>(wrow + min(kn + u * SK_KSTEP + 32 * g + 8 * c, k_last));
+                    a[u][c] = *reinterpret_cast<const bf16x8*>(wrow + min(kk + u * SK_KSTEP + 8 * g + 32 * c, k_last));
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u) {
+                // x_s holds zeros from c_end to the padded end of the chunk
+                const bool live = kk + u * SK_KSTEP < c_begin + chunk;
+                const __bf16* xk = xp + min(kk + u * SK_KSTEP, c_begin + chunk - SK_KSTEP);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
-                    // x_s holds zeros from c_end to the padded end of the chunk
-                    const bf16x8 b = *reinterpret_cast<const bf16x8*>(xp + min(kk + u * SK_KSTEP, c_begin + chunk - SK_KSTEP) + 8 * c);
-                    const bool live = kk + u * SK_KSTEP < c_begin + chunk;
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][c], live ? b : zero8(), acc, 0, 0, 0);
+#pragma unroll
+                    for (int b = 0; b < MB; ++b) {
+                        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xk + b * 16 * xs_stride + 32 * c);
+                        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][c], live ? xb : zero8(), acc[b], 0, 0, 0);
+                    }
                 }
             }
         }
     }
     if (!active) return;
-    // acc[i] = y[m = col][n = n0 + 4*g + i]
+    // acc[b][i] = y[m = 16 * b + col][n = n0 + 4*g + i]
     const int n = n0 + 4 * g;
-    const int m = col;
-    if (m >= M) return;
-    if (!direct) {
-        float* p = partial + ((int64_t)split * M + m) * N + n;
-        if (n + 3 < N && (N % 4) == 0) {
-            *reinterpret_cast<f32x4*>(p) = acc;
-        } else {
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+        const int m = 16 * b + col;
+        if (m >= M) continue;
+        if (!direct) {
+            float* p = partial + ((int64_t)split * M + m) * N + n;
+            if (n + 3 < N && (N % 4) == 0) {
+                *reinterpret_cast<f32x4*>(p) = acc[b];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < N) p[i] = acc[b][i];
+            }
+        } else if (y_is_f32) {
+            float* p = (float*)y + (int64_t)m * y_stride + n;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (n + i < N) p[i] = acc[i];
+                if (n + i < N) p[i] = acc[b][i];
+        } else {
+            __bf16* p = (__bf16*)y + (int64_t)m * y_stride + n;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (n + i < N) p[i] = (__bf16)acc[b][i];
         }
-    } else if (y_is_f32) {
-        float* p = (float*)y + (int64_t)m * y_stride + n;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (n + i < N) p[i] = acc[i];
-    } else {
-        __bf16* p = (__bf16*)y + (int64_t)m * y_stride + n;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (n + i < N) p[i] = (__bf16)acc[i];
     }
 }
 
@@ -166,9 +176,9 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
                                       float* scratch, int splits, int defer_finish, int64_t M, int64_t N,
                                       int64_t K, int* splits_used, hipStream_t stream) {
     if (M == 0 || N == 0) return 0;
-    if (M < 0 || M > 16 || K % 8 || K <= 0 || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
-        nva_fail("linear_skinny: needs 1..16 rows, K %% 8 == 0 and 16-byte aligned rows (M=%lld K=%lld)", (long long)M,
-                 (long long)K);
+    if (M < 0 || M > SK_MAX_ROWS || K % 8 || K <= 0 || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
+        nva_fail("linear_skinny: needs 1..%d rows, K %% 8 == 0 and 16-byte aligned rows (M=%lld K=%lld)", SK_MAX_ROWS,
+                 (long long)M, (long long)K);
         return 1;
     }
     if (N > 0x7fffffff || K > 0x7fffffff || splits < 1 || splits > 65535) return nva_fail("linear_skinny: bad sizes");
@@ -179,10 +189,23 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     kps = (kps + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
     const int real_splits = (int)((K + kps - 1) / kps);
     const int64_t tiles = (N + 15) / 16;
-    dim3 grid((unsigned)((tiles + SK_WAVES - 1) / SK_WAVES), (unsigned)real_splits);
-    const size_t lds = (size_t)16 * ((kps < SK_CHUNK ? kps : SK_CHUNK) + 8) * sizeof(__bf16);
-    hipLaunchKernelGGL(linear_skinny_kernel, grid, dim3(SK_WAVES * NVA_WAVE), lds, stream, (const __bf16*)x, x_stride,
-                       (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32, direct, (int)M, (int)N, (int)K, kps);
+#define LAUNCH(MB)                                                                                                     \
+    do {                                                                                                               \
+        constexpr int waves = SkShape<MB>::waves;                                                                      \
+        dim3 grid((unsigned)((tiles + waves - 1) / waves), (unsigned)real_splits);                                     \
+        const size_t lds = (size_t)16 * MB * ((kps < SkShape<MB>::chunk ? kps : SkShape<MB>::chunk) + 8) * sizeof(__bf16); \
+        static const hipError_t lds_allowed = hipFuncSetAttribute(                                                     \
+            (const void*)linear_skinny_kernel<MB>, hipFuncAttributeMaxDynamicSharedMemorySize,                         \
+            16 * MB * (SkShape<MB>::chunk + 8) * (int)sizeof(__bf16));                                                 \
+        if (lds_allowed != hipSuccess) return nva_fail("linear_skinny: %s", hipGetErrorString(lds_allowed));           \
+        hipLaunchKernelGGL(linear_skinny_kernel<MB>, grid, dim3(waves * NVA_WAVE), lds, stream, (const __bf16*)x,      \
+                           x_stride, (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32, direct, (int)M,       \
+                           (int)N, (int)K, kps);                                                                       \
+    } while (0)
+    if (M <= 16) LAUNCH(1);
+    else if (M <= 32) LAUNCH(2);
+    else LAUNCH(4);
+#undef LAUNCH
     if (splits_used) *splits_used = real_splits;
     int rc = nva_check_launch("linear_skinny");
     // deferred: the partial sums [real_splits][M][N] stay in scratch for a kernel that consumes them

@@ -102,7 +102,9 @@ class HipKernels:
         # bit 0: a token id outside the vocabulary; bit 1: a visible key without a page
         self.fault_flag = torch.zeros(1, dtype=torch.int32, device=self.device)
         # Rows up to which the bfloat16 product runs on the engine's own kernels.
-        self.own_matmul_rows = 16
+        self.own_matmul_rows = 16           # bfloat16 products with more rows go to the library ...
+        self.skinny_max_rows = 64           # ... unless the weight is small (see _own_rows); the kernel's limit
+        self.small_weight_bytes = 64 << 20
         self.skinny_target_waves = 2048     # the k range of a few-row product is split until this many waves run
         self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
@@ -234,16 +236,18 @@ class HipKernels:
             raise KernelError("linear: bias does not fit")
         out_dtype = torch.float32 if out_float32 else x.dtype
         if x.dtype == torch.bfloat16 and self._skinny_takes(x, xs, weight, ws, k):
-            if deferred and 0 < m <= self.own_matmul_rows and not out_float32 and out is None and self.fuse_split_sums:
+            own = 0 < m <= self._own_rows(n, k)
+            if deferred and own and not out_float32 and out is None and self.fuse_split_sums:
                 return self._linear_skinny(x, xs, weight, ws, bias, None, 0, False, False, m, n, k, defer=True)
-            if m <= self.own_matmul_rows or out_float32:
+            if own or out_float32:
                 if out is None:
                     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
                 om, on, os_ = _rows2d(out, "linear output")
                 if (om, on) != (m, n) or out.dtype != out_dtype:
                     raise KernelError("linear: output does not match")
-                for r0 in range(0, m, 16):          # more rows (logits of many places): 16 at a time
-                    r1 = min(m, r0 + 16)
+                rows = self.skinny_max_rows      # more rows (logits of many places): that many at a time
+                for r0 in range(0, m, rows):
+                    r1 = min(m, r0 + rows)
                     self._linear_skinny(x[r0:r1], xs, weight, ws, bias, out[r0:r1], os_, out_float32, False, r1 - r0, n, k)
                 return out
         if x.dtype == torch.bfloat16 and not out_float32:
@@ -262,12 +266,21 @@ class HipKernels:
                      c_i64(m), c_i64(n), c_i64(k), self._stream())
         return out
 
+    def _own_rows(self, n: int, k: int) -> int:
+        """Up to how many rows of x the weight-streaming kernel takes a bfloat16 product of this
+        weight; beyond, the library product runs.  Measured on the layer shapes of an 8B model:
+        up to 16 rows the kernel is as fast or faster for every weight; up to 64 rows only for
+        small weights, where the library's kernels leave the GPU half empty."""
+        if 2 * n * k <= self.small_weight_bytes:
+            return self.skinny_max_rows
+        return self.own_matmul_rows
+
     @staticmethod
     def _skinny_takes(x, xs, weight, ws, k) -> bool:
         return k % 8 == 0 and xs % 8 == 0 and ws % 8 == 0 and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
 
     def _linear_skinny(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k, defer=False):
-        """The weight-streaming kernel for at most 16 rows; k is split over workgroups when the
+        """The weight-streaming kernel for at most 64 rows; k is split over workgroups when the
         output is too narrow to fill the GPU.  defer: the partial sums are returned as a SplitSum
         (or the finished tensor, where k is not split)."""
         tiles = (n + 15) // 16
@@ -293,7 +306,7 @@ class HipKernels:
         m, k, xs = _rows2d(x, "linear input")
         n, wk, ws = _rows2d(weight, "linear weight")
         if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
-                0 < m <= self.own_matmul_rows and self._skinny_takes(x, xs, weight, ws, k):
+                0 < m <= self._own_rows(n, k) and self._skinny_takes(x, xs, weight, ws, k):
             out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
             self._linear_skinny(x, xs, weight, ws, None, out, n // 2, False, True, m, n, k)
             return out

@@ -137,7 +137,7 @@ def test_linear_bfloat16(hip, ref, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (8, 6144, 4096), (64, 320, 12288), (17, 1000, 264), (33, 24, 8),
-                                   (5, 130, 72)])
+                                   (5, 130, 72), (48, 40000, 1288), (20, 40004, 2304), (64, 4096, 4096)])
 def test_linear_bfloat16_few_rows_streams_the_weights(hip, ref, m, n, k):
     """The decode-step product (few rows, k split over workgroups) against a double product."""
     x, w = _rand((m, k), torch.bfloat16, 21), _rand((n, k), torch.bfloat16, 22, 0.05)
