@@ -210,61 +210,64 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 }
 
 // Merges the splits of one (token, head): o = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m).
-// One wave per (token, head).  The (max, sum) pairs of up to 64 splits are read by 64 lanes at
-// once; the partial outputs are then read four splits at a time so that the loads overlap.
-__global__ void __launch_bounds__(NVA_WAVE)
+// One workgroup of four waves per (token, head).  Every wave finds the maximum m over the visible
+// splits, then takes every fourth group of four splits (their loads overlap) and the four partial
+// sums meet in LDS; the order of the sum depends on the number of splits only.
+#define MERGE_WAVES 4
+__global__ void __launch_bounds__(MERGE_WAVES * NVA_WAVE)
 attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                          __bf16* __restrict__ out, int64_t out_stride, const int32_t* __restrict__ positions,
                          int num_q_heads, int head_dim, int window, int split_len, int num_splits) {
+    __shared__ float acc_s[MERGE_WAVES][4 * NVA_WAVE];
+    __shared__ float l_s[MERGE_WAVES];
     const int64_t t = blockIdx.x;
-    const int head = blockIdx.y, lane = threadIdx.x;
+    const int head = blockIdx.y, lane = threadIdx.x % NVA_WAVE, wave = threadIdx.x / NVA_WAVE;
     const int pos = positions[t];
     const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
     const int s_lo = first / split_len, s_hi = pos / split_len;          // splits that hold visible keys
     const int64_t slot0 = ((int64_t)t * num_q_heads + head) * num_splits;
     float m = -INFINITY;
-    for (int s0 = s_lo; s0 <= s_hi; s0 += NVA_WAVE) {
-        const int s = s0 + lane;
-        m = fmaxf(m, s <= s_hi ? part_ml[(slot0 + s) * 2] : -INFINITY);
-    }
+    for (int s = s_lo + lane; s <= s_hi; s += NVA_WAVE) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
     m = wave_max(m);
     float l = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = s_lo; s0 <= s_hi; s0 += NVA_WAVE) {
-        const int s = s0 + lane;
-        float w = 0.f;
-        if (s <= s_hi) {
+    for (int s0 = s_lo + 4 * wave; s0 <= s_hi; s0 += 4 * MERGE_WAVES) {
+        float wj[4], v[4][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int s = min(s0 + j, s_hi);                              // a split past the end: read again, weight 0
             const float ms = part_ml[(slot0 + s) * 2];
-            w = (ms == -INFINITY) ? 0.f : __expf(ms - m);
-            l += part_ml[(slot0 + s) * 2 + 1] * w;
-        }
-        const int count = min(NVA_WAVE, s_hi - s0 + 1);
-        for (int j0 = 0; j0 < count; j0 += 4) {
-            float wj[4], v[4][4];
+            wj[j] = (s0 + j > s_hi || ms == -INFINITY) ? 0.f : __expf(ms - m);
+            l += part_ml[(slot0 + s) * 2 + 1] * wj[j];
+            const float* po = part_o + (slot0 + s) * head_dim;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                wj[j] = __shfl(w, min(j0 + j, NVA_WAVE - 1), NVA_WAVE);
-                if (j0 + j >= count) wj[j] = 0.f;
-                const float* po = part_o + (slot0 + s0 + min(j0 + j, count - 1)) * head_dim;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int d = lane + i * NVA_WAVE;
-                    v[j][i] = d < head_dim ? po[d] : 0.f;
-                }
+            for (int i = 0; i < 4; ++i) {
+                const int d = lane + i * NVA_WAVE;
+                v[j][i] = d < head_dim ? po[d] : 0.f;
             }
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] += v[j][i] * wj[j];
         }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += v[j][i] * wj[j];
     }
-    l = wave_sum(l);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc_s[wave][lane + i * NVA_WAVE] = acc[i];
+    if (lane == 0) l_s[wave] = l;
+    __syncthreads();
+    if (wave != 0) return;
+    l = 0.f;
+#pragma unroll
+    for (int w = 0; w < MERGE_WAVES; ++w) l += l_s[w];
     const float inv = l > 0.f ? 1.f / l : 0.f;
     __bf16* orow = out + t * out_stride + (int64_t)head * head_dim;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int d = lane + i * NVA_WAVE;
-        if (d < head_dim) orow[d] = (__bf16)(acc[i] * inv);
+        float o = 0.f;
+#pragma unroll
+        for (int w = 0; w < MERGE_WAVES; ++w) o += acc_s[w][d];
+        if (d < head_dim) orow[d] = (__bf16)(o * inv);
     }
 }
 
@@ -316,7 +319,7 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     if (rc) return rc;
     if (num_splits > 1) {
         dim3 mgrid((unsigned)tokens, (unsigned)num_q_heads);
-        hipLaunchKernelGGL(attn_decode_merge_kernel, mgrid, dim3(NVA_WAVE), 0, stream, part_o, part_ml, (__bf16*)out,
+        hipLaunchKernelGGL(attn_decode_merge_kernel, mgrid, dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, (__bf16*)out,
                            out_stride, positions, num_q_heads, head_dim, window, split_len, num_splits);
         rc = nva_check_launch("attn_decode_merge");
     }
