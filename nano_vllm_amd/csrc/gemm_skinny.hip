@@ -37,7 +37,9 @@ __device__ __forceinline__ bf16x8 zero8() {
     return z;
 }
 
-// direct: 1 = the only split writes y itself (as bfloat16 or float); 0 = float partials [split][M][N]
+// direct: 0 = float partials [split][M][N]; 1 = the only split writes y itself (as bfloat16 or
+// float); 2 = the same for W = [gate rows; up rows]: a wave then takes 8 gate rows and the 8 up rows
+// that belong to them, and writes silu(gate) * up, [M][N / 2].
 //
 // The workgroup's waves share one range of k, so its slice of x (16 * MB rows, rows >= M zero) is
 // staged once in LDS (row stride padded by 16 bytes against bank conflicts).
@@ -57,9 +59,13 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     const int chunk = min(k_per_split, SkShape<MB>::chunk);
     const int xs_stride = chunk + 8;
 
-    const int n0 = (blockIdx.x * WAVES + wave) * 16;
-    const bool active = n0 < N;                       // idle waves still help to stage x
-    const __bf16* wrow = w + (int64_t)min(n0 + col, N - 1) * w_stride;
+    const bool gated = direct == 2;
+    const int inner = N / 2;
+    const int tile = blockIdx.x * WAVES + wave;
+    const int n0 = gated ? tile * 8 : tile * 16;
+    const bool active = n0 < (gated ? inner : N);     // idle waves still help to stage x
+    const int w_row = gated ? min(n0 + (col & 7), inner - 1) + (col >= 8 ? inner : 0) : min(n0 + col, N - 1);
+    const __bf16* wrow = w + (int64_t)w_row * w_stride;
     f32x4 acc[MB];
 #pragma unroll
     for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -110,6 +116,27 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
         }
     }
     if (!active) return;
+    if (gated) {
+        // acc[b][i] of lanes g < 2 is the gate of y[m = 16 * b + col][j = n0 + 4*g + i], the same register
+        // of lane + 32 its up; both are rounded to bfloat16 before the gating as the reference's
+        // projection is (activation.py:8-11)
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            const int m = 16 * b + col;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float up = (float)(__bf16)__shfl(acc[b][i], (lane + 32) % NVA_WAVE, NVA_WAVE);
+                const float gate = (float)(__bf16)acc[b][i];
+                const int j = n0 + 4 * g + i;
+                if (g < 2 && m < M && j < inner) {
+                    const float v = gate / (1.f + __expf(-gate)) * up;
+                    if (y_is_f32) ((float*)y)[(int64_t)m * y_stride + j] = v;
+                    else ((__bf16*)y)[(int64_t)m * y_stride + j] = (__bf16)v;
+                }
+            }
+        }
+        return;
+    }
     // acc[b][i] = y[m = 16 * b + col][n = n0 + 4*g + i]
     const int n = n0 + 4 * g;
 #pragma unroll
@@ -183,12 +210,12 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     }
     if (N > 0x7fffffff || K > 0x7fffffff || splits < 1 || splits > 65535) return nva_fail("linear_skinny: bad sizes");
     if (swiglu && (N % 2)) return nva_fail("linear_skinny: the gated form needs an even number of weight rows");
-    const int direct = splits == 1 && !bias && !swiglu && !defer_finish;
+    const int direct = splits == 1 && !bias && !defer_finish ? (swiglu ? 2 : 1) : 0;
     if (!direct && !scratch) return nva_fail("linear_skinny: this call needs scratch memory");
     int kps = (int)((K + splits - 1) / splits);
     kps = (kps + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
     const int real_splits = (int)((K + kps - 1) / kps);
-    const int64_t tiles = (N + 15) / 16;
+    const int64_t tiles = direct == 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
 #define LAUNCH(MB)                                                                                                     \
     do {                                                                                                               \
         constexpr int waves = SkShape<MB>::waves;                                                                      \

@@ -285,11 +285,13 @@ class HipKernels:
         (or the finished tensor, where k is not split)."""
         tiles = (n + 15) // 16
         splits = max(1, min((self.skinny_target_waves + tiles - 1) // tiles, k // 256))
+        if swiglu and bias is None and 2 * tiles >= self.skinny_target_waves:
+            splits = 1          # wide enough without a split of k: the gating happens in the product kernel
         if defer and splits == 1:
             defer = False
             out = torch.empty((m, n), dtype=x.dtype, device=x.device)
             os_ = n
-        direct = splits == 1 and bias is None and not swiglu
+        direct = splits == 1 and bias is None
         scratch = None if direct else torch.empty(splits * m * n, dtype=torch.float32, device=x.device)
         used = ctypes.c_int(0)
         library.call("gemm_skinny", "bf16", "nva_linear_skinny", _p(x), c_i64(xs), _p(weight), c_i64(ws),

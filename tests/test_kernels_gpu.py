@@ -152,7 +152,8 @@ def test_linear_bfloat16_few_rows_streams_the_weights(hip, ref, m, n, k):
     _close(hip[torch.bfloat16].linear(x, w, b), (want + b.double()).float().to(torch.bfloat16), torch.bfloat16)
 
 
-@pytest.mark.parametrize("m,inner,k", [(1, 12288, 4096), (8, 200, 96), (64, 160, 256), (100, 64, 128)])
+@pytest.mark.parametrize("m,inner,k", [(1, 12288, 4096), (8, 200, 96), (64, 160, 256), (100, 64, 128), (5, 8196, 264),
+                                       (40, 9004, 1288), (16, 12288, 4096)])
 def test_linear_silu_mul(hip, ref, m, inner, k):
     x, w = _rand((m, k), torch.bfloat16, 24), _rand((2 * inner, k), torch.bfloat16, 25, 0.1)
     _close(hip[torch.bfloat16].linear_silu_mul(x, w), ref.linear_silu_mul(x, w), torch.bfloat16)
