@@ -22,13 +22,12 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 #define SK_UNROLL 2
 #define SK_MAX_ROWS 64
 
-// Row blocks of x (MB), waves per workgroup and the k of x staged at a time: the LDS slice is
-// 16 * MB rows * (chunk + 8) * 2 bytes.  More rows of x take more waves per workgroup, so that a
-// staged slice of x serves more rows of W, and a shorter chunk, so that two workgroups fit a CU.
+// Row blocks of x (MB) and waves per workgroup: more rows of x take more waves, so that a staged
+// slice of x serves more rows of W.
 template <int MB> struct SkShape;
-template <> struct SkShape<1> { static constexpr int waves = 4, chunk = 1536; };
-template <> struct SkShape<2> { static constexpr int waves = 8, chunk = 1024; };
-template <> struct SkShape<4> { static constexpr int waves = 8, chunk = 512; };
+template <> struct SkShape<1> { static constexpr int waves = 4; };
+template <> struct SkShape<2> { static constexpr int waves = 8; };
+template <> struct SkShape<4> { static constexpr int waves = 8; };
 
 __device__ __forceinline__ bf16x8 zero8() {
     bf16x8 z;
@@ -41,22 +40,28 @@ __device__ __forceinline__ bf16x8 zero8() {
 // float); 2 = the same for W = [gate rows; up rows]: a wave then takes 8 gate rows and the 8 up rows
 // that belong to them, and writes silu(gate) * up, [M][N / 2].
 //
-// The workgroup's waves share one range of k, so its slice of x (16 * MB rows, rows >= M zero) is
-// staged once in LDS (row stride padded by 16 bytes against bank conflicts).
+// The workgroup's waves share one range of k, so its slice of x is staged in LDS, `chunk` columns
+// at a time (a multiple of 256; row stride padded by 16 bytes against bank conflicts): the M rows
+// and one row of zeros, which the MFMA columns beyond M read.  Lane (row, g) takes the 16-byte piece
+// g + 4c of its row's 256 bytes in load c, so that one load instruction covers 64 contiguous bytes
+// of each of the wave's 16 rows; x is read from LDS at the same k.  The loads of a step of 256 k
+// are issued at its top and the products wait for them one by one: the other waves of the CU cover
+// the latency, so many short waves (a finer split of k) run faster than few long ones.  A chunk's
+// first loads are issued before its slice of x is staged.  Only a ragged last step (K % 256) moves
+// its offsets back into the row: what it reads beyond K meets zeros of x_s.
 template <int MB>
 __global__ void __launch_bounds__(SkShape<MB>::waves * NVA_WAVE)
 linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf16* __restrict__ w, int64_t w_stride,
                      float* __restrict__ partial, void* __restrict__ y, int64_t y_stride, int y_is_f32, int direct,
-                     int M, int N, int K, int k_per_split) {
+                     int M, int N, int K, int k_per_split, int chunk) {
     constexpr int WAVES = SkShape<MB>::waves;
-    constexpr int ROWS = 16 * MB;
-    extern __shared__ __attribute__((aligned(16))) __bf16 x_s[];     // [ROWS][chunk + 8]
+    constexpr int STEP = SK_KSTEP * SK_UNROLL;
+    extern __shared__ __attribute__((aligned(16))) __bf16 x_s[];     // [M + 1][chunk + 8]
     const int wave = threadIdx.x / NVA_WAVE, lane = threadIdx.x % NVA_WAVE;
     const int col = lane & 15, g = lane >> 4;
     const int split = blockIdx.y;
     const int k_begin = split * k_per_split;
     const int k_end = min(K, k_begin + k_per_split);
-    const int chunk = min(k_per_split, SkShape<MB>::chunk);
     const int xs_stride = chunk + 8;
 
     const bool gated = direct == 2;
@@ -67,21 +72,31 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     const int w_row = gated ? min(n0 + (col & 7), inner - 1) + (col >= 8 ? inner : 0) : min(n0 + col, N - 1);
     const __bf16* wrow = w + (int64_t)w_row * w_stride;
     f32x4 acc[MB];
+    const __bf16* xrow[MB];
 #pragma unroll
-    for (int b = 0; b < MB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
-
-    // Lane (row, g) takes the 16-byte piece g + 4c of its row's 256 bytes in load c, so that one load
-    // instruction covers 64 contiguous bytes of each of the wave's 16 rows; x is read from LDS at the
-    // same k.  Every load of W is unconditional (an offset past the end of the row is moved back into
-    // it: what it reads meets zeros of x_s or is dropped).  The loads of a step are issued at its top
-    // and the products wait for them one by one; other waves of the CU cover the latency.  (Loads
-    // issued a step ahead were measured slower, and they read past the split's range of k.)
+    for (int b = 0; b < MB; ++b) {
+        acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+        xrow[b] = x_s + min(col + 16 * b, M) * xs_stride + 8 * g;
+    }
     const int k_last = K - 8;
+    bf16x8 a[SK_UNROLL][4];
+
+#define SK_LOAD_CLAMPED(kk)                                                                                            \
+    _Pragma("unroll") for (int u = 0; u < SK_UNROLL; ++u) _Pragma("unroll") for (int c = 0; c < 4; ++c)                \
+        a[u][c] = *reinterpret_cast<const bf16x8*>(wrow + min((kk) + u * SK_KSTEP + 8 * g + 32 * c, k_last))
+#define SK_PRODUCTS(off)                                                                                               \
+    _Pragma("unroll") for (int u = 0; u < SK_UNROLL; ++u) _Pragma("unroll") for (int c = 0; c < 4; ++c)                \
+        _Pragma("unroll") for (int b = 0; b < MB; ++b)                                                                 \
+            acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(                                                          \
+                a[u][c], *reinterpret_cast<const bf16x8*>(xrow[b] + (off) + u * SK_KSTEP + 32 * c), acc[b], 0, 0, 0)
+
     for (int c_begin = k_begin; c_begin < k_end; c_begin += chunk) {
         const int c_end = min(k_end, c_begin + chunk);
-        // ---- stage x[0:ROWS][c_begin:c_begin + chunk] (zeros beyond M and c_end)
+        const int len = c_end - c_begin;
+        SK_LOAD_CLAMPED(c_begin);
+        // ---- stage x[0:M][c_begin:c_begin + chunk] and the zero row (zeros beyond c_end as well)
         __syncthreads();
-        for (int idx = threadIdx.x; idx < ROWS * (chunk / 8); idx += WAVES * NVA_WAVE) {
+        for (int idx = threadIdx.x; idx < (M + 1) * (chunk / 8); idx += WAVES * NVA_WAVE) {
             const int m = idx / (chunk / 8), piece = idx % (chunk / 8);
             const int k = c_begin + piece * 8;
             bf16x8 v = zero8();
@@ -90,31 +105,24 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
         }
         __syncthreads();
         if (!active) continue;
-        const __bf16* xp = x_s + col * xs_stride + 8 * g - c_begin;
-
-        for (int kk = c_begin; kk < c_end; kk += SK_KSTEP * SK_UNROLL) {
-            bf16x8 a[SK_UNROLL][4];
+        SK_PRODUCTS(0);
+        const int full = len / STEP;
+        const bf16x8* wp = reinterpret_cast<const bf16x8*>(wrow + c_begin + 8 * g);
+        int s = 1;
+        for (; s < full; ++s) {
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u)
 #pragma unroll
-                for (int c = 0; c < 4; ++c)
-                    a[u][c] = *reinterpret_cast<const bf16x8*>(wrow + min(kk + u * SK_KSTEP + 8 * g + 32 * c, k_last));
-#pragma unroll
-            for (int u = 0; u < SK_UNROLL; ++u) {
-                // x_s holds zeros from c_end to the padded end of the chunk
-                const bool live = kk + u * SK_KSTEP < c_begin + chunk;
-                const __bf16* xk = xp + min(kk + u * SK_KSTEP, c_begin + chunk - SK_KSTEP);
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-#pragma unroll
-                    for (int b = 0; b < MB; ++b) {
-                        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xk + b * 16 * xs_stride + 32 * c);
-                        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][c], live ? xb : zero8(), acc[b], 0, 0, 0);
-                    }
-                }
-            }
+                for (int c = 0; c < 4; ++c) a[u][c] = wp[(s * STEP + u * SK_KSTEP + 32 * c) / 8];
+            SK_PRODUCTS(s * STEP);
+        }
+        if (s * STEP < len) {
+            SK_LOAD_CLAMPED(c_begin + s * STEP);
+            SK_PRODUCTS(s * STEP);
         }
     }
+#undef SK_LOAD_CLAMPED
+#undef SK_PRODUCTS
     if (!active) return;
     if (gated) {
         // acc[b][i] of lanes g < 2 is the gate of y[m = 16 * b + col][j = n0 + 4*g + i], the same register
@@ -197,7 +205,7 @@ linear_skinny_finish_kernel(const float* __restrict__ partial, int splits, const
 
 // splits: how many ranges k is cut into (>= 1); scratch must hold splits * M * N floats when
 // splits > 1 or a bias, swiglu or defer_finish is asked for.  splits_used receives the number of
-// ranges really used (k per range is rounded up to a multiple of 128).  Returns 1 for shapes this kernel does not take.
+// ranges really used (k per range is rounded up to a multiple of 256).  Returns 1 for shapes this kernel does not take.
 NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
                                       const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
                                       float* scratch, int splits, int defer_finish, int64_t M, int64_t N,
@@ -213,21 +221,21 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     const int direct = splits == 1 && !bias && !defer_finish ? (swiglu ? 2 : 1) : 0;
     if (!direct && !scratch) return nva_fail("linear_skinny: this call needs scratch memory");
     int kps = (int)((K + splits - 1) / splits);
-    kps = (kps + SK_KSTEP - 1) / SK_KSTEP * SK_KSTEP;
+    kps = (kps + SK_KSTEP * SK_UNROLL - 1) / (SK_KSTEP * SK_UNROLL) * (SK_KSTEP * SK_UNROLL);
     const int real_splits = (int)((K + kps - 1) / kps);
     const int64_t tiles = direct == 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
+    // columns of x staged at a time: about 36 KB of LDS for the M + 1 rows, so that several workgroups fit a CU
+    int chunk = (36864 / (2 * ((int)M + 1)) - 8) / 256 * 256;
+    chunk = chunk < 256 ? 256 : chunk > 2048 ? 2048 : chunk;
+    if (chunk > kps) chunk = kps;
+    const size_t lds = (size_t)(M + 1) * (chunk + 8) * sizeof(__bf16);
 #define LAUNCH(MB)                                                                                                     \
     do {                                                                                                               \
         constexpr int waves = SkShape<MB>::waves;                                                                      \
         dim3 grid((unsigned)((tiles + waves - 1) / waves), (unsigned)real_splits);                                     \
-        const size_t lds = (size_t)16 * MB * ((kps < SkShape<MB>::chunk ? kps : SkShape<MB>::chunk) + 8) * sizeof(__bf16); \
-        static const hipError_t lds_allowed = hipFuncSetAttribute(                                                     \
-            (const void*)linear_skinny_kernel<MB>, hipFuncAttributeMaxDynamicSharedMemorySize,                         \
-            16 * MB * (SkShape<MB>::chunk + 8) * (int)sizeof(__bf16));                                                 \
-        if (lds_allowed != hipSuccess) return nva_fail("linear_skinny: %s", hipGetErrorString(lds_allowed));           \
         hipLaunchKernelGGL(linear_skinny_kernel<MB>, grid, dim3(waves * NVA_WAVE), lds, stream, (const __bf16*)x,      \
                            x_stride, (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32, direct, (int)M,       \
-                           (int)N, (int)K, kps);                                                                       \
+                           (int)N, (int)K, kps, chunk);                                                                \
     } while (0)
     if (M <= 16) LAUNCH(1);
     else if (M <= 32) LAUNCH(2);

@@ -105,7 +105,7 @@ class HipKernels:
         self.own_matmul_rows = 16           # bfloat16 products with more rows go to the library ...
         self.skinny_max_rows = 64           # ... unless the weight is small (see _own_rows); the kernel's limit
         self.small_weight_bytes = 64 << 20
-        self.skinny_target_waves = 2048     # the k range of a few-row product is split until this many waves run
+        self.skinny_target_waves = 4096     # the k range of a few-row product is split until this many waves run
         self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
         self.mfma_attention = True
@@ -284,8 +284,10 @@ class HipKernels:
         output is too narrow to fill the GPU.  defer: the partial sums are returned as a SplitSum
         (or the finished tensor, where k is not split)."""
         tiles = (n + 15) // 16
-        splits = max(1, min((self.skinny_target_waves + tiles - 1) // tiles, k // 256))
-        if swiglu and bias is None and 2 * tiles >= self.skinny_target_waves:
+        # many rows of x: the partial sums weigh more, and the waves do more work each
+        target = self.skinny_target_waves if m <= 16 else self.skinny_target_waves // 2
+        splits = max(1, min((target + tiles - 1) // tiles, k // 256))
+        if swiglu and bias is None and 2 * tiles >= target:
             splits = 1          # wide enough without a split of k: the gating happens in the product kernel
         if defer and splits == 1:
             defer = False
