@@ -28,15 +28,18 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 #define PF_BN 64
 #define PF_WAVES 4
 
+struct Masked { static constexpr bool value = true; };     // a tile that the window's start or the diagonal cuts
+struct Whole { static constexpr bool value = false; };     // a tile every row of the workgroup sees whole
+
 template <int D>
 // two waves per SIMD (at most 256 registers) up to head_dim 128; beyond that the accumulators need more
 __global__ void __launch_bounds__(PF_WAVES * NVA_WAVE, D <= 128 ? 2 : 1)
 attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
                     const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                     const int32_t* __restrict__ block_tables, int table_stride,
-                    const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens, int first_seq,
-                    int num_seqs, int num_q_heads, int num_kv_heads, int page_size, float scale, int window,
-                    int32_t* error_flag) {
+                    const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens,
+                    const int32_t* __restrict__ tiles, int num_tiles, int resident, int num_q_heads, int num_kv_heads,
+                    int page_size, float scale, int window, int32_t* error_flag) {
     constexpr int KS = D + 8;             // K tile row stride (elements): 16 bytes of padding against bank conflicts
     constexpr int VS = PF_BN + 8;         // V tile row stride
     constexpr int DC = D / 16;            // 16-channel steps of the first product
@@ -44,14 +47,22 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     __shared__ __attribute__((aligned(16))) __bf16 k_s[PF_BN * KS];
     __shared__ __attribute__((aligned(16))) __bf16 v_s[D * VS];
 
-    // ---- which request and which 32 rows of it
-    int seq = first_seq, tile = blockIdx.x;
-    for (; seq < num_seqs; ++seq) {
-        const int tiles = (cu_seqlens_q[seq + 1] - cu_seqlens_q[seq] + PF_BM - 1) / PF_BM;
-        if (tile < tiles) break;
-        tile -= tiles;
+    // ---- which request, which 32 rows of it, which heads.  `tiles` lists (request, row tile) from the
+    // most keys to the fewest; a rank counts (tile, head chunk) pairs in that order.  Workgroups are
+    // handed out in the order of their index, to the XCDs in turn and within an XCD to its CUs in turn:
+    // with more workgroups than fit the GPU at once, the heaviest go first and the light ones fill the
+    // gaps; with fewer, the first half of the indices takes the heavy ranks in order and the second half
+    // the light ranks from the lightest, so that a CU's two workgroups are a heavy and a light one.
+    const int ny = num_kv_heads * ((num_q_heads / num_kv_heads + PF_WAVES - 1) / PF_WAVES);
+    const int total = num_tiles * ny;
+    const int L = blockIdx.x;
+    int rank = L;
+    if (total <= resident) {
+        const int heavy = 8 * ((total + 15) / 16);
+        rank = L < heavy ? L : total - 1 - (L - heavy);
     }
-    if (seq >= num_seqs) return;
+    const int by = rank % ny;
+    const int seq = tiles[2 * (rank / ny)], tile = tiles[2 * (rank / ny) + 1];
     const int q_begin = cu_seqlens_q[seq];
     const int q_len = cu_seqlens_q[seq + 1] - q_begin;
     const int kv_len = kv_lens[seq];
@@ -62,7 +73,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     const int vt = nva_v_tile(page_size);
     const int G = num_q_heads / num_kv_heads;
     const int chunks = (G + PF_WAVES - 1) / PF_WAVES;
-    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int kvh = by / chunks, chunk = by % chunks;
     const int tid = threadIdx.x, wave = tid / NVA_WAVE, lane = tid % NVA_WAVE;
     const int col = lane & 31, h = lane >> 5;
     const int head_in_group = chunk * PF_WAVES + wave;
@@ -124,6 +135,11 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     // a key outside the visible range is replaced by the nearest visible one (its scores are masked by
     // the key index; V is zeroed when it is written to LDS, in the tiles at the two ends only).  The
     // loads of tile t + 1 are issued before the products of tile t.
+    //
+    // The tiles fall into three runs: those the window's start cuts, those every row sees whole, and
+    // those the diagonal cuts.  The middle run, most of a long prompt, runs without any masking, and
+    // where pages hold whole tiles (page_size % 64 == 0) its loads are one base address per tile, held
+    // in scalar registers, plus an offset per thread that never changes.
     constexpr int PIECES = PF_BN * (D / 8) / (PF_WAVES * NVA_WAVE);
     static_assert(PF_BN * (D / 8) % (PF_WAVES * NVA_WAVE) == 0, "the tile divides over the threads");
     const int last_key = kb_hi - 1;
@@ -148,10 +164,27 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
             v_reg[i] = *reinterpret_cast<const bf16x8*>(vb + nva_v_offset(key0 % page_size, d, D, vt));
         }
     };
-    issue_loads(kb_lo);
+    // a tile that lies whole in one page and is visible whole: kb % 64 == 0, page_size % 64 == 0
+    const int k_thread = (tid / (D / 8)) * D + (tid % (D / 8)) * 8;                 // + i * rows_per_pass * D
+    constexpr int K_PASS = (PF_WAVES * NVA_WAVE / (D / 8)) * D;
+    const int v_thread = (((tid % 8) / 4) * D + tid / 8) * 32 + ((tid % 8) % 4) * 8;   // + i * 32 channels * 32
+    constexpr int V_PASS = (PF_WAVES * NVA_WAVE / (PF_BN / 8)) * 32;
+    auto issue_loads_fast = [&](int kb) {
+        const int page = __builtin_amdgcn_readfirstlane(table_s[kb / page_size - page_lo]);
+        const int kip = kb % page_size;
+        const __bf16* kbase = k_cache + (((int64_t)page * num_kv_heads + kvh) * page_size + kip) * D;
+        const __bf16* vbase = v_cache + ((int64_t)page * num_kv_heads + kvh) * D * (int64_t)page_size + (int64_t)(kip / 32) * D * 32;
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) k_reg[i] = *reinterpret_cast<const bf16x8*>(kbase + k_thread + i * K_PASS);
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i) v_reg[i] = *reinterpret_cast<const bf16x8*>(vbase + v_thread + i * V_PASS);
+    };
+    // (the split of a thread's pieces into a fixed offset and a step per pass needs 256 % (D / 8) == 0)
+    const bool fast_pages = page_size % PF_BN == 0 && (PF_WAVES * NVA_WAVE) % (D / 8) == 0;
 
-    for (int kb = kb_lo; kb < kb_hi; kb += PF_BN) {
-        // ---- registers -> LDS
+    // One tile: registers -> LDS, the next tile's loads, scores, softmax, second product.
+    auto round = [&](int kb, auto masked_tag, int next_kb, bool next_fast) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) {
             const int idx = tid + i * PF_WAVES * NVA_WAVE;
@@ -161,7 +194,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         {
             const int grp = tid % (PF_BN / 8);
             const int key0 = kb + grp * 8;
-            const bool edge = kb < first_any || kb + PF_BN > kb_hi;          // the same for the whole workgroup
+            const bool edge = MASKED && (kb < first_any || kb + PF_BN > kb_hi);  // the same for the whole workgroup
 #pragma unroll
             for (int i = 0; i < PIECES; ++i) {
                 const int d = tid / (PF_BN / 8) + i * (PF_WAVES * NVA_WAVE / (PF_BN / 8));
@@ -175,7 +208,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
             }
         }
         __syncthreads();
-        issue_loads(min(kb + PF_BN, last_key & ~(PF_BN - 1)));               // after the last tile: read again, dropped
+        if (next_fast) issue_loads_fast(next_kb);
+        else issue_loads(next_kb);
 
         if (active) {
             // ---- scores of 2 x 32 keys
@@ -194,9 +228,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
             // this lane: query `col`; register e of tile kt is key kb + 32*kt + 16*(e/8) + 8*h + e%8.
             // The maximum is taken of the raw scores (scale > 0) and the scale folded, with log2(e),
             // into the exponent: p = 2^((s - m) * scale * log2 e), one fused multiply-add per score.
-            const bool full = kb + PF_BN - 1 <= start + q0 && kb >= first_any + (window > 0 ? PF_BM : 0);
             float m_new = m_run;
-            if (!full) {
+            if (MASKED) {
 #pragma unroll
                 for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -251,7 +284,24 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
             }
         }
         __syncthreads();
+    };
+
+    // whole tiles: kb in [whole_lo, whole_hi)
+    const int whole_lo = window > 0 ? (first_any + PF_BM + PF_BN - 1) & ~(PF_BN - 1) : kb_lo;
+    const int whole_hi = (start + q0 + 1) & ~(PF_BN - 1);
+    const int a_end = min(max(whole_lo, kb_lo), (kb_hi + PF_BN - 1) & ~(PF_BN - 1));
+    const int b_end = max(a_end, min(whole_hi, kb_hi));
+    const int after_last = last_key & ~(PF_BN - 1);                      // after the last tile: read again, dropped
+    if (a_end < b_end && fast_pages && kb_lo == a_end) issue_loads_fast(kb_lo);
+    else issue_loads(kb_lo);
+    int kb = kb_lo;
+    for (; kb < a_end; kb += PF_BN) round(kb, Masked(), min(kb + PF_BN, after_last), false);
+    for (; kb < b_end - PF_BN; kb += PF_BN) round(kb, Whole(), kb + PF_BN, fast_pages);
+    if (kb < b_end) {
+        round(kb, Whole(), min(kb + PF_BN, after_last), false);
+        kb += PF_BN;
     }
+    for (; kb < kb_hi; kb += PF_BN) round(kb, Masked(), min(kb + PF_BN, after_last), false);
 
     // acc[mt][4a + b] = O[query col][channel 32*mt + 8a + 4h + b]
     if (!active || !row_ok) return;
@@ -268,15 +318,16 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         }
 }
 
-// total_tiles = sum over requests first_seq.. of ceil(q_len / 32), computed by the caller.
+// tiles: int32 [num_tiles][2] = (request, row tile of 32 queries) for every tile of the step's
+// portions, ordered from the most visible keys to the fewest (the caller builds it once per step).
 // Returns 1 (and leaves a message) for shapes this kernel does not take.
 NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride,
                                      const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                      int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,
-                                     int first_seq, int num_seqs, int64_t total_tiles, int num_q_heads,
+                                     const int32_t* tiles, int64_t num_tiles, int num_q_heads,
                                      int num_kv_heads, int head_dim, int page_size, float scale, int window,
                                      int32_t* error_flag, hipStream_t stream) {
-    if (total_tiles == 0 || first_seq >= num_seqs) return 0;
+    if (num_tiles == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_prefill: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
     if (head_dim % 32 || head_dim < 32 || head_dim > 256 || page_size % 8 || page_size <= 0) {
@@ -286,19 +337,27 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
     }
     const int G = num_q_heads / num_kv_heads;
     const int64_t grid_y = (int64_t)num_kv_heads * ((G + PF_WAVES - 1) / PF_WAVES);
-    if (total_tiles < 0 || total_tiles > 0x7fffffff || grid_y > 65535 || window < 0 || table_stride <= 0)
-        return nva_fail("attn_prefill: bad sizes (tiles %lld, heads %lld)", (long long)total_tiles, (long long)grid_y);
+    if (!tiles || num_tiles < 0 || num_tiles * grid_y > 0x7fffffff || window < 0 || table_stride <= 0)
+        return nva_fail("attn_prefill: bad sizes (tiles %lld, heads %lld)", (long long)num_tiles, (long long)grid_y);
     if (table_stride > 4096) {
         nva_fail("attn_prefill: block tables of %d pages do not fit the kernel's staging buffer", table_stride);
         return 1;
     }
     const size_t table_bytes = (size_t)table_stride * sizeof(int32_t);
-    dim3 grid((unsigned)total_tiles, (unsigned)grid_y);
+    // workgroups the GPU holds at once: two per CU (the kernel's registers allow no more)
+    static int resident = 0;
+    if (!resident) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            return nva_fail("attn_prefill: cannot read the number of CUs");
+        resident = 2 * cus;
+    }
+    dim3 grid((unsigned)(num_tiles * grid_y));
 #define LAUNCH(DD)                                                                                                 \
     hipLaunchKernelGGL(attn_prefill_kernel<DD>, grid, dim3(PF_WAVES * NVA_WAVE), table_bytes, stream, (const __bf16*)q, \
                        q_stride, (__bf16*)out, out_stride, (const __bf16*)k_cache, (const __bf16*)v_cache,           \
-                       block_tables, table_stride, cu_seqlens_q, kv_lens, first_seq, num_seqs, num_q_heads,          \
-                       num_kv_heads, page_size, scale, window, error_flag)
+                       block_tables, table_stride, cu_seqlens_q, kv_lens, tiles, (int)num_tiles, resident,           \
+                       num_q_heads, num_kv_heads, page_size, scale, window, error_flag)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;

@@ -13,6 +13,8 @@ from typing import Hashable, List, Optional, Sequence
 
 import torch
 
+from ..kernels.ops import prefill_tile_order
+
 
 @dataclass
 class StepEntry:
@@ -41,6 +43,7 @@ class StepBatch:
     seq_starts: torch.Tensor         # int32 [S] tokens each request had in the cache before
     state_slots: torch.Tensor        # int32 [S]
     logits_rows: Optional[torch.Tensor]   # int32 [R] flat token indices, in the caller's order
+    prefill_tiles: Optional[torch.Tensor]  # int32 [tiles, 2]: (request, 32-row tile) of the portions, most keys first
     groups: List[GroupBatch]
     max_q_len: int
     max_kv_len: int
@@ -119,8 +122,10 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
         if max(widths, default=1) > table_width:
             raise ValueError(f"a block table of {max(widths)} pages exceeds the fixed width {table_width}")
         widths = [table_width] * num_groups
+    num_decode = sum(1 for n in q_lens if n == 1)
+    tile_order = prefill_tile_order(q_lens, starts, num_decode)
     flat: List[int] = []
-    flat += input_ids + positions + token_seq + cu + kv_lens + starts + state_slots + rows
+    flat += input_ids + positions + token_seq + cu + kv_lens + starts + state_slots + rows + tile_order
     for g in range(num_groups):
         flat += slot_maps[g]
         for tb in tables[g]:
@@ -145,13 +150,14 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
     b_ids, b_pos, b_seq = take(T), take(T), take(T)
     b_cu, b_kv, b_starts, b_slots = take(S + 1), take(S), take(S), take(S)
     b_rows = take(len(rows)) if rows else None
+    b_tiles = take(len(tile_order)).view(-1, 2) if tile_order else None
     groups = []
     for g in range(num_groups):
         sm = take(T)
         bt = take(S * widths[g]).view(S, widths[g])
         groups.append(GroupBatch(bt, sm))
     return StepBatch(
-        num_tokens=T, num_seqs=S, num_decode=sum(1 for n in q_lens if n == 1),
+        num_tokens=T, num_seqs=S, num_decode=num_decode, prefill_tiles=b_tiles,
         input_ids=b_ids, positions=b_pos, token_seq=b_seq, cu_seqlens_q=b_cu, kv_lens=b_kv,
         seq_starts=b_starts, state_slots=b_slots, logits_rows=b_rows, groups=groups,
         max_q_len=max(q_lens), max_kv_len=max(kv_lens), q_lens=q_lens, starts=starts,

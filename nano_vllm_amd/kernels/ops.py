@@ -85,6 +85,22 @@ def _t(x):
     return x.tensor() if isinstance(x, SplitSum) else x
 
 
+PREFILL_ROWS = 32       # query rows of one workgroup of the prefill attention kernel
+
+
+def prefill_tile_order(q_lens, starts, first_seq: int) -> list:
+    """Flat [(request, row tile), ...] of the requests from `first_seq` on, from the tile that
+    sees the most keys to the one that sees the fewest: the prefill attention kernel hands its
+    workgroups out in this order, so that the long ones start first."""
+    units = []
+    for s in range(first_seq, len(q_lens)):
+        n = q_lens[s]
+        for t in range((n + PREFILL_ROWS - 1) // PREFILL_ROWS):
+            units.append((starts[s] + min(n, (t + 1) * PREFILL_ROWS), s, t))
+    units.sort(key=lambda u: (-u[0], u[1], u[2]))
+    return [v for u in units for v in (u[1], u[2])]
+
+
 class HipKernels:
     """Every device operation of the engine.  Needs a GPU and the compiled libraries."""
 
@@ -444,10 +460,18 @@ class HipKernels:
         if start < tokens and q.dtype == torch.bfloat16 and self.mfma_attention and start == batch.num_decode and \
                 self._decode_kernel_takes(1, head_dim, page_size, q, qs, out, os_):
             # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
-            tiles = sum((n + 31) // 32 for n in batch.q_lens[batch.num_decode:])
+            tiles = getattr(batch, "prefill_tiles", None)
+            if tiles is None:       # a batch that was not built by the engine: order the tiles here, once
+                flat = prefill_tile_order(batch.q_lens, batch.starts if getattr(batch, "starts", None) else
+                                          [int(kv) - n for kv, n in zip(batch.kv_lens.tolist(), batch.q_lens)],
+                                          batch.num_decode)
+                tiles = torch.tensor(flat, dtype=torch.int32, device=q.device).view(-1, 2)
+                batch.prefill_tiles = tiles
+            if tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 2 or not tiles.is_contiguous():
+                raise KernelError("attention: prefill_tiles must be contiguous int32 [tiles, 2]")
             library.call("attn_prefill", "bf16", "nva_attn_prefill", _p(q), c_i64(qs), _p(out), c_i64(os_), _p(k_cache),
                          _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q), _p(batch.kv_lens),
-                         c_i32(batch.num_decode), c_i32(batch.num_seqs), c_i64(tiles), c_i32(num_heads),
+                         _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
                          _p(self.fault_flag), self._stream())
             start = tokens
