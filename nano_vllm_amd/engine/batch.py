@@ -11,6 +11,7 @@ from __future__ import annotations
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..kernels.ops import prefill_tile_order
@@ -73,10 +74,12 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
     T, S = t, len(entries)
     num_groups = len(cache.groups)
 
+    # per request a few arrays (a portion of a prompt has thousands of tokens: no Python per token)
     input_ids, positions, token_seq = [], [], []
     cu, kv_lens, starts, state_slots, q_lens = [0], [], [], [], []
     slot_maps = [[] for _ in range(num_groups)]
     tables = [[] for _ in range(num_groups)]
+    one_ids, one_pos, one_slots = [], [], [[] for _ in range(num_groups)]
     seen = set()
     for s, i in enumerate(order):
         e = entries[i]
@@ -90,26 +93,42 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
         if e.start < 0 or e.start + n > rc.num_tokens:
             raise ValueError(f"request {e.request!r}: positions {e.start}..{e.start + n - 1} are not reserved "
                              f"in the cache ({rc.num_tokens} are)")
-        for tok in e.tokens:
-            if not 0 <= tok < vocab_size:
-                raise ValueError(f"request {e.request!r}: token id {tok} is outside the vocabulary of {vocab_size}")
-        input_ids.extend(e.tokens)
-        positions.extend(range(e.start, e.start + n))
-        token_seq.extend([s] * n)
         cu.append(cu[-1] + n)
         kv_lens.append(e.start + n)
         starts.append(e.start)
         q_lens.append(n)
         state_slots.append(rc.state_slot)
+        if n == 1:                                   # a decoded token (these come first): plain integers
+            tok = e.tokens[0]
+            if not 0 <= tok < vocab_size:
+                raise ValueError(f"request {e.request!r}: token id {tok} is outside the vocabulary of {vocab_size}")
+            one_ids.append(tok)
+            one_pos.append(e.start)
+            for g in range(num_groups):
+                table = rc.tables[g]
+                tables[g].append(table)
+                page = table[e.start // page_size]
+                if page < 0:
+                    raise ValueError(f"request {e.request!r}: position {e.start} has no page in group {g}")
+                one_slots[g].append(page * page_size + e.start % page_size)
+            continue
+        toks = np.asarray(e.tokens, dtype=np.int64)
+        if toks.ndim != 1 or int(toks.min()) < 0 or int(toks.max()) >= vocab_size:
+            bad = next(int(tok) for tok in e.tokens if not 0 <= tok < vocab_size)
+            raise ValueError(f"request {e.request!r}: token id {bad} is outside the vocabulary of {vocab_size}")
+        pos = np.arange(e.start, e.start + n, dtype=np.int64)
+        input_ids.append(toks)
+        positions.append(pos)
+        token_seq.append(np.full(n, s, dtype=np.int64))
         for g in range(num_groups):
             table = rc.tables[g]
             tables[g].append(table)
-            sm = slot_maps[g]
-            for pos in range(e.start, e.start + n):
-                page = table[pos // page_size]
-                if page < 0:
-                    raise ValueError(f"request {e.request!r}: position {pos} has no page in group {g}")
-                sm.append(page * page_size + pos % page_size)
+            pages = np.asarray(table, dtype=np.int64)[pos // page_size]
+            if int(pages.min()) < 0:
+                where = int(pos[int(np.argmax(pages < 0))])
+                raise ValueError(f"request {e.request!r}: position {where} has no page in group {g}")
+            slot_maps[g].append(pages * page_size + pos % page_size)
+    num_decode = len(one_ids)
     rows = []
     for i, e in enumerate(entries):
         for w in e.want:
@@ -122,15 +141,28 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
         if max(widths, default=1) > table_width:
             raise ValueError(f"a block table of {max(widths)} pages exceeds the fixed width {table_width}")
         widths = [table_width] * num_groups
-    num_decode = sum(1 for n in q_lens if n == 1)
     tile_order = prefill_tile_order(q_lens, starts, num_decode)
-    flat: List[int] = []
-    flat += input_ids + positions + token_seq + cu + kv_lens + starts + state_slots + rows + tile_order
-    for g in range(num_groups):
-        flat += slot_maps[g]
-        for tb in tables[g]:
-            flat += tb + [-1] * (widths[g] - len(tb))
-    host = torch.tensor(flat, dtype=torch.int32)
+    scalars = cu + kv_lens + starts + state_slots + rows + tile_order
+    if num_decode == S:                              # decoded tokens only: one list, one conversion
+        flat: List[int] = one_ids + one_pos + list(range(S)) + scalars
+        for g in range(num_groups):
+            flat += one_slots[g]
+            for tb in tables[g]:
+                flat += tb
+                flat += [-1] * (widths[g] - len(tb))
+        host = torch.tensor(flat, dtype=torch.int32)
+    else:
+        as_array = lambda values: np.asarray(values, dtype=np.int64)
+        pieces = [as_array(one_ids)] + input_ids + [as_array(one_pos)] + positions
+        pieces += [np.arange(num_decode, dtype=np.int64)] + token_seq + [as_array(scalars)]
+        for g in range(num_groups):
+            pieces += [as_array(one_slots[g])] + slot_maps[g]
+            padded: List[int] = []
+            for tb in tables[g]:
+                padded += tb
+                padded += [-1] * (widths[g] - len(tb))
+            pieces.append(as_array(padded))
+        host = torch.from_numpy(np.concatenate(pieces).astype(np.int32))
     if static is not None:
         if static.numel() != host.numel():
             raise ValueError("the static batch buffer does not fit this batch's layout")
