@@ -138,6 +138,120 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, PartialInput part, T* q_ou
     }
 }
 
+// The same work for many tokens at once (portions of prompts).  A workgroup of 256 threads takes
+// one head of 256 / LPH consecutive tokens, LPH = head_dim / 16 lanes per token: a lane holds the
+// eight elements 8p.. of the head's first half and the eight of its second half that pair with them,
+// so every access is a 16-byte (32-byte in float) vector and the norm's sum crosses LPH lanes only.
+// A v head goes through LDS, and where 32 tokens in a row have 32 slots in a row that start a key
+// tile of the V cache, a lane writes eight keys of one channel at once.
+template <typename T, int LPH>
+__global__ void __launch_bounds__(256)
+qk_norm_rope_store_tile_kernel(T* qkv, int64_t row_stride, int tokens, int num_q_heads, int num_kv_heads,
+                               const void* __restrict__ q_weight, const void* __restrict__ k_weight, int w_is_f32,
+                               float eps, const float* __restrict__ table, const int32_t* __restrict__ positions,
+                               const int32_t* __restrict__ slots, T* k_cache, T* v_cache, int page_size) {
+    constexpr int D = 16 * LPH, HALF = 8 * LPH, TB = 256 / LPH, VS = TB + 8 / (int)sizeof(T) * 2;
+    __shared__ __attribute__((aligned(16))) T v_s[D * VS];
+    __shared__ int run_ok[(TB + 31) / 32];
+    const int tid = threadIdx.x, r = tid / LPH, p = tid % LPH;
+    const int head = blockIdx.y;
+    const int t0 = blockIdx.x * TB, t = t0 + r;
+    const bool live = t < tokens;
+    T* row = qkv + (int64_t)(live ? t : 0) * row_stride + (int64_t)head * D;
+    const int64_t slot = live && slots ? slots[t] : -1;
+    float x1[8], x2[8];
+    load8(row + 8 * p, x1);
+    load8(row + HALF + 8 * p, x2);
+
+    if (head >= num_q_heads + num_kv_heads) {                       // a v head
+        if (!v_cache) return;
+        const int h = head - num_q_heads - num_kv_heads;
+        const int vt = nva_v_tile(page_size);
+        // runs of 32 tokens whose slots are 32 in a row from the start of a key tile
+        if (tid < (TB + 31) / 32) run_ok[tid] = vt == 32 ? 1 : 0;
+        __syncthreads();
+        const int run = r / 32;
+        const int64_t run_slot = (t0 + run * 32 < tokens && slots) ? slots[t0 + run * 32] : -1;
+        if (!(live && run_slot >= 0 && run_slot % 32 == 0 && slot == run_slot + r % 32)) run_ok[run] = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            v_s[(8 * p + e) * VS + r] = from_float<T>(x1[e]);
+            v_s[(HALF + 8 * p + e) * VS + r] = from_float<T>(x2[e]);
+        }
+        __syncthreads();
+        // pieces of eight keys of one channel: TB / 8 per channel
+        for (int idx = tid; idx < D * (TB / 8); idx += 256) {
+            const int d = idx / (TB / 8), piece = idx % (TB / 8);
+            const int tok = piece * 8;                               // first token of the piece within the block
+            if (run_ok[tok / 32]) {
+                const int64_t s0 = slots[t0 + (tok & ~31)];
+                const int64_t page = s0 / page_size, off = s0 % page_size + (tok & 31);
+                T* dst = v_cache + ((page * num_kv_heads + h) * (int64_t)D) * page_size + nva_v_offset((int)off, d, D, vt);
+                float v[8];
+                load8(&v_s[d * VS + tok], v);
+                store8(dst, v);
+            } else {
+                for (int e = 0; e < 8; ++e) {
+                    const int tt = t0 + tok + e;
+                    const int64_t se = tt < tokens && slots ? slots[tt] : -1;
+                    if (se < 0) continue;
+                    const int64_t page = se / page_size, off = se % page_size;
+                    v_cache[((page * num_kv_heads + h) * (int64_t)D) * page_size + nva_v_offset((int)off, d, D, vt)] =
+                        v_s[d * VS + tok + e];
+                }
+            }
+        }
+        return;
+    }
+
+    const bool is_q = head < num_q_heads;
+    const void* weight = is_q ? q_weight : k_weight;
+    if (weight) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ss += x1[e] * x1[e] + x2[e] * x2[e];
+#pragma unroll
+        for (int o = LPH / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, NVA_WAVE);
+        const float scale = rsqrtf(ss / (float)D + eps);
+        float w1[8], w2[8];
+        if (w_is_f32) {
+            load8((const float*)weight + 8 * p, w1);
+            load8((const float*)weight + HALF + 8 * p, w2);
+        } else {
+            load8((const T*)weight + 8 * p, w1);
+            load8((const T*)weight + HALF + 8 * p, w2);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            x1[e] = round_through<T>(round_through<T>(x1[e] * scale) * w1[e]);
+            x2[e] = round_through<T>(round_through<T>(x2[e] * scale) * w2[e]);
+        }
+    }
+    if (table) {
+        const float* angles = table + (int64_t)(live ? positions[t] : 0) * D;
+        float c[8], sn[8];
+        load8(angles + 8 * p, c);
+        load8(angles + HALF + 8 * p, sn);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float y1 = x1[e] * c[e] - x2[e] * sn[e];
+            const float y2 = x2[e] * c[e] + x1[e] * sn[e];
+            x1[e] = y1;
+            x2[e] = y2;
+        }
+    }
+    if (!live) return;
+    store8(row + 8 * p, x1);
+    store8(row + HALF + 8 * p, x2);
+    if (!is_q && slot >= 0 && k_cache) {
+        const int h = head - num_q_heads;
+        const int64_t page = slot / page_size, off = slot % page_size;
+        T* dst = k_cache + ((page * num_kv_heads + h) * (int64_t)page_size + off) * D;
+        store8(dst + 8 * p, x1);
+        store8(dst + HALF + 8 * p, x2);
+    }
+}
+
 static int launch_qk(elem_t* qkv, int64_t row_stride, PartialInput part, elem_t* q_out, int64_t q_out_stride,
                      int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, const void* q_weight,
                      const void* k_weight, int w_is_f32, float eps, const float* table, const int32_t* positions,
@@ -153,6 +267,29 @@ static int launch_qk(elem_t* qkv, int64_t row_stride, PartialInput part, elem_t*
         return nva_fail("qk_norm_rope_store: a cache needs a page size and slots");
     if (table && !positions) return nva_fail("qk_norm_rope_store: a rotation table needs positions");
     const int total = num_q_heads + 2 * num_kv_heads;
+    // many tokens of a finished projection: the tiled kernel, where the head size has an instance
+    // and the rows can be read in vectors
+    const int lph = head_dim / 16;
+    if (!part.sums && tokens >= 64 && head_dim % 16 == 0 && (lph & (lph - 1)) == 0 && lph <= 16 && total <= 65535 &&
+        row_stride % 8 == 0 && nva_aligned(qkv, 32) && (!q_weight || nva_aligned(q_weight, 32)) &&
+        (!k_weight || nva_aligned(k_weight, 32)) && nva_aligned(table, 32) && nva_aligned(k_cache, 32) &&
+        nva_aligned(v_cache, 32)) {
+        const int tb = 256 / lph;
+        dim3 tgrid((unsigned)((tokens + tb - 1) / tb), (unsigned)total);
+#define TILE(LPH)                                                                                                      \
+    hipLaunchKernelGGL((qk_norm_rope_store_tile_kernel<elem_t, LPH>), tgrid, dim3(256), 0, stream, qkv, row_stride,   \
+                       (int)tokens, num_q_heads, num_kv_heads, q_weight, k_weight, w_is_f32, eps, table, positions,  \
+                       slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size)
+        switch (lph) {
+            case 1: TILE(1); break;
+            case 2: TILE(2); break;
+            case 4: TILE(4); break;
+            case 8: TILE(8); break;
+            default: TILE(16); break;
+        }
+#undef TILE
+        return nva_check_launch("qk_norm_rope_store_tile");
+    }
     const int waves = 4;
     dim3 grid((unsigned)tokens, (total + waves - 1) / waves);
     hipLaunchKernelGGL(qk_norm_rope_store_kernel<elem_t>, grid, dim3(waves * NVA_WAVE), 0, stream, qkv, row_stride, part,

@@ -242,6 +242,39 @@ def test_qk_norm_rope_store(hip, ref, dtype, hq, hkv, D, page, norm):
     assert torch.equal(c, qkv)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,D,page", [(4, 2, 16, 8), (3, 1, 32, 32), (6, 2, 64, 64), (8, 2, 128, 256),
+                                           (2, 2, 256, 32), (5, 5, 48, 16), (4, 1, 128, 24)])
+def test_qk_norm_rope_store_of_a_long_portion(hip, ref, dtype, hq, hkv, D, page):
+    """Many tokens take the tiled kernel: slots in a row from the start of a key tile (written
+    eight keys at a time), slots in a row from the middle of one, scattered slots, tokens that
+    are not stored, and a last block that is not full."""
+    T = 331
+    pages = (T + 416 + page - 1) // page + 6                        # slots 0..415 hold the runs
+    k = hip[dtype]
+    qkv = _rand((T, (hq + 2 * hkv) * D), dtype, 41)
+    qw, kw = _rand((D,), dtype, 42) + 1, _rand((D,), dtype, 43) + 1
+    table = ref.rotary_table(_inv_freq(D, 1e6), 700)
+    positions = torch.randint(0, 700, (T,), dtype=torch.int32, device=DEV)
+    slots = torch.randperm(pages * page - 416)[:T] + 416            # scattered, beyond the runs
+    slots[0:128] = torch.arange(128, 256)                           # in a row from the start of a tile
+    slots[128:230] = torch.arange(5, 5 + 102)                       # in a row from the middle of a tile
+    slots[256:320] = torch.arange(256 + 96, 256 + 160)              # another run that starts at a tile
+    slots[17] = -1
+    slots[300] = -1
+    slots = slots.to(torch.int32).to(DEV)
+    assert len(set(slots.tolist()) - {-1}) == T - 2
+    caches = [new_caches(pages, hkv, D, page, dtype, DEV) for _ in range(2)]
+    a, b = qkv.clone(), qkv.clone()
+    qa = k.qk_norm_rope_store(a, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[0])
+    qb = ref.qk_norm_rope_store(b, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[1])
+    _close(qa, qb, dtype, "q")
+    _close(a, b, dtype, "k in place")
+    _close(caches[0][0], caches[1][0], dtype, "k cache")
+    assert torch.equal(caches[0][1], caches[1][1])                  # values are copied as they are
+    assert torch.equal(a[:, (hq + hkv) * D:], qkv[:, (hq + hkv) * D:])
+
+
 def test_qk_refusals(hip):
     from nano_vllm_amd.kernels import KernelError
     k = hip[torch.float32]
