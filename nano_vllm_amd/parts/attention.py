@@ -84,7 +84,6 @@ class Attention(Part):
         # deferred: the products below are handed to the q/k preparation and to the block's norm only
         pe = self.position_encoding
         table = pe.rotary_table() if pe is not None else None
-        # deferred: the products below are handed to the q/k preparation and to the block's norm only
         qkv = k.linear(x, w["qkv_proj.weight"], w.get("qkv_proj.bias"), deferred=pe is None or table is not None)
         group = batch.groups[cache.group]
         slots = None if self.shared else group.slot_mapping

@@ -272,3 +272,161 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     lost = r.step([StepEntry("a", reqs["a"][10:], 10, list(range(20)))]).cpu()
     r.cache.release("a")
     assert H.rel_err(lost, whole["a"][10:]) > 1e-3
+
+
+# ------------------------------------------------------------------------------ toy feed-forward with routing,
+# ------------------------------------------------------------------------------ toy position encoding
+class ToyRoutedFeedForward(Part):
+    """Each token goes to its top_k of E small experts (up -> silu -> down), mixed with the softmax
+    of the chosen router logits.  The router runs in float32.  Products on the chosen rows go through
+    the package's own linear kernel; the routing is plain torch."""
+
+    def __init__(self, params, build):
+        super().__init__(params, build)
+        self.hidden, self.inner = params["hidden_size"], params["inner"]
+        self.experts, self.top_k = params["experts"], params["top_k"]
+
+    def param_decls(self):
+        d = {"router.weight": ParamDecl((self.experts, self.hidden), dtype="float32")}
+        for e in range(self.experts):
+            d[f"experts.{e}.up.weight"] = ParamDecl((self.inner, self.hidden))
+            d[f"experts.{e}.down.weight"] = ParamDecl((self.hidden, self.inner))
+        return d
+
+    def forward(self, x, batch=None):
+        w = self.weights
+        scores = x.float() @ w["router.weight"].float().T
+        top, chosen = scores.topk(self.top_k, dim=-1)
+        mix = torch.softmax(top, dim=-1)
+        out = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+        for e in range(self.experts):
+            rows, slot = (chosen == e).nonzero(as_tuple=True)
+            if rows.numel() == 0:
+                continue
+            h = self.kernels.linear(x[rows].contiguous(), w[f"experts.{e}.up.weight"])
+            h = (h.float() * torch.sigmoid(h.float())).to(x.dtype)
+            y = self.kernels.linear(h, w[f"experts.{e}.down.weight"])
+            out.index_add_(0, rows, y.float() * mix[rows, slot, None])
+        return out.to(x.dtype)
+
+
+class ToyInterleavedRotary(Part):
+    """Rotation of the pairs (2i, 2i+1) (the package's own encoding pairs i with i + D/2): no
+    table, so the mixer calls apply()."""
+
+    def __init__(self, params, build):
+        super().__init__(params, build)
+        self.head_dim, self.theta = params["head_dim"], params["theta"]
+
+    def rotary_table(self):
+        return None
+
+    def apply(self, q, k, positions, num_heads, num_kv_heads, head_dim):
+        inv = 1.0 / (self.theta ** (torch.arange(0, head_dim, 2, dtype=torch.float32, device=q.device) / head_dim))
+        ang = positions.float()[:, None] * inv[None, :]
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        for x, heads in ((q, num_heads), (k, num_kv_heads)):
+            if heads == 0:
+                continue
+            v = x.float().reshape(x.shape[0], heads, head_dim // 2, 2)
+            a, b = v[..., 0], v[..., 1]
+            x.copy_(torch.stack((a * cos - b * sin, b * cos + a * sin), dim=-1).reshape(x.shape[0], -1).to(x.dtype))
+
+
+def _routed_spec(cfg: dict) -> ModelSpec:
+    H_, V, D = cfg["hidden_size"], cfg["vocab_size"], cfg["head_dim"]
+    norm = PartSpec("rms_norm", {"dim": H_, "eps": cfg["eps"]})
+    dense = PartSpec("swiglu", {"hidden_size": H_, "intermediate_size": cfg["inner"]})
+    routed = PartSpec("toy_routed", {"hidden_size": H_, "inner": cfg["expert_inner"], "experts": cfg["experts"],
+                                     "top_k": cfg["top_k"]})
+    attn = PartSpec("attention", {"hidden_size": H_, "num_heads": cfg["heads"], "num_kv_heads": cfg["kv_heads"],
+                                  "head_dim": D, "qk_norm": True, "eps": cfg["eps"], "position_encoding": "pairs",
+                                  "window": None})
+    names = {"mixer_norm": "norm1", "mixer": "attn", "feed_forward_norm": "norm2", "feed_forward": "ffn"}
+    layers = tuple(LayerSpec(PartSpec("pre_norm_residual"), {"mixer_norm": norm, "mixer": attn, "feed_forward_norm": norm,
+                                                              "feed_forward": f}, f"layers.{i}", names)
+                   for i, f in enumerate([routed, dense, routed]))
+    return ModelSpec(architecture="ToyRoutedLM", hidden_size=H_, vocab_size=V, max_position=256, dtype="float32",
+                     embedding=PartSpec("token_embedding", {"name": "embed"}), layers=layers,
+                     order=tuple(LayerRun(i) for i in range(3)),
+                     final_norm=PartSpec("rms_norm", {"dim": H_, "eps": cfg["eps"], "name": "norm"}),
+                     head=PartSpec("output_head", {"name": "head", "tied": False}),
+                     position_encodings={"pairs": PartSpec("toy_pairs_rotary", {"head_dim": D, "theta": cfg["theta"]})})
+
+
+def _routed_plain(w, cfg, tokens, first_position=0):
+    """The toy model on a whole sequence, in double, written without the package."""
+    f = lambda name: w[name].double()
+    H_, D, hq, hkv = cfg["hidden_size"], cfg["head_dim"], cfg["heads"], cfg["kv_heads"]
+    eps = cfg["eps"]
+    norm = lambda x, name: x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * f(name)
+    T = len(tokens)
+    pos = torch.arange(first_position, first_position + T, dtype=torch.float64)
+    inv = 1.0 / (cfg["theta"] ** (torch.arange(0, D, 2, dtype=torch.float64) / D))
+    ang = pos[:, None] * inv[None, :]
+
+    def rotate(x):                                                  # [T, heads, D], pairs (2i, 2i+1)
+        v = x.reshape(T, -1, D // 2, 2)
+        a, b = v[..., 0], v[..., 1]
+        c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        return torch.stack((a * c - b * s, b * c + a * s), dim=-1).reshape(T, -1, D)
+
+    x = f("embed.weight")[torch.tensor(tokens)]
+    for i in range(3):
+        p = f"layers.{i}"
+        h = norm(x, f"{p}.norm1.weight")
+        q = (h @ f(f"{p}.attn.q_proj.weight").T).reshape(T, hq, D)
+        k = (h @ f(f"{p}.attn.k_proj.weight").T).reshape(T, hkv, D)
+        v = (h @ f(f"{p}.attn.v_proj.weight").T).reshape(T, hkv, D)
+        q = rotate(norm(q, f"{p}.attn.q_norm.weight"))
+        k = rotate(norm(k, f"{p}.attn.k_norm.weight"))
+        k, v = k.repeat_interleave(hq // hkv, 1), v.repeat_interleave(hq // hkv, 1)
+        s = torch.einsum("thd,shd->hts", q, k) * D ** -0.5
+        s = s.masked_fill(torch.ones(T, T).triu(1).bool(), float("-inf"))
+        o = torch.einsum("hts,shd->thd", torch.softmax(s, -1), v).reshape(T, hq * D)
+        x = x + o @ f(f"{p}.attn.o_proj.weight").T
+        h = norm(x, f"{p}.norm2.weight")
+        if i == 1:
+            g = h @ f(f"{p}.ffn.gate_proj.weight").T
+            y = (g * torch.sigmoid(g) * (h @ f(f"{p}.ffn.up_proj.weight").T)) @ f(f"{p}.ffn.down_proj.weight").T
+        else:
+            top, chosen = (h @ f(f"{p}.ffn.router.weight").T).topk(cfg["top_k"], dim=-1)
+            mix = torch.softmax(top, -1)
+            y = torch.zeros_like(h)
+            for t in range(T):
+                for j in range(cfg["top_k"]):
+                    e = int(chosen[t, j])
+                    u = f(f"{p}.ffn.experts.{e}.up.weight") @ h[t]
+                    y[t] += mix[t, j] * (f(f"{p}.ffn.experts.{e}.down.weight") @ (u * torch.sigmoid(u)))
+        x = x + y
+    return (norm(x, "norm.weight") @ f("head.weight").T).float()
+
+
+def test_a_toy_feed_forward_with_routing_and_another_position_encoding(tmp_path):
+    """Both are defined above, registered here and run through loader, step function and cache
+    like the package's own parts; the result is checked against a computation in double that
+    shares nothing with the package."""
+    from safetensors.torch import load_file
+    register_part("feed_forward", "toy_routed", ToyRoutedFeedForward, replace=True)
+    register_part("position_encoding", "toy_pairs_rotary", ToyInterleavedRotary, replace=True)
+    register_architecture("ToyRoutedLM", lambda d: d, _routed_spec, replace=True)
+    cfg = {"architectures": ["ToyRoutedLM"], "hidden_size": 72, "vocab_size": 131, "inner": 88, "expert_inner": 40,
+           "experts": 5, "top_k": 2, "heads": 6, "kv_heads": 2, "head_dim": 16, "eps": 1e-5, "theta": 5e3,
+           "torch_dtype": "float32"}
+    folder = write_random_model(str(tmp_path / "routed"), cfg, seed=8, std=0.15)
+    r = ModelRunner.from_folder(folder, dtype="float32", page_size=8, num_pages=24, max_requests=3, quiet=True)
+    w = load_file(os.path.join(folder, "model.safetensors"))
+    assert w["layers.0.ffn.router.weight"].dtype == torch.float32 and "layers.2.ffn.experts.4.down.weight" in w
+    reqs = {k: H.random_tokens(131, n, 20 + i) for i, (k, n) in enumerate({"a": 45, "b": 70, "c": 23}.items())}
+    want = {k: _routed_plain(w, cfg, v) for k, v in reqs.items()}
+    got = H.run_portions(r, "a", reqs["a"], [45])
+    assert H.rel_err(got, want["a"]) < 2e-5
+    got = H.run_portions(r, "b", reqs["b"], H.changing_portions(70, 4))
+    assert H.rel_err(got, want["b"]) < 2e-5
+    mixed = H.run_mixed(r, reqs, seed=3)
+    for k in reqs:
+        assert H.rel_err(mixed[k], want[k]) < 2e-5, k
+    # only distances count: all positions shifted by 40 give the same logits
+    shifted = _routed_plain(w, cfg, reqs["c"], first_position=40)
+    assert H.rel_err(shifted, want["c"]) < 1e-9
+    r.kernels.check_faults()
