@@ -4,6 +4,7 @@ options those of SamplingParams (nanovllm/sampling_params.py:4-11).
 
     python -m nano_vllm_amd.cli generate --model DIR --prompt-ids 1,2,3 [--prompt "text"] ...
     python -m nano_vllm_amd.cli random-model --config config.json --seed 0 --out DIR
+    python -m nano_vllm_amd.cli throughput --model DIR [--random-weights SEED] --num-seqs 256 ...
 """
 from __future__ import annotations
 
@@ -25,6 +26,8 @@ def add_engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--schedule", default="prefill_first", choices=["prefill_first", "mixed"])
     ap.add_argument("--no-prefix-caching", action="store_true")
+    ap.add_argument("--random-weights", type=int, default=None, metavar="SEED",
+                    help="draw the weights on the device from this seed: the folder needs config.json only")
 
 
 def engine_kwargs(args) -> dict:
@@ -32,7 +35,8 @@ def engine_kwargs(args) -> dict:
                 max_model_len=args.max_model_len, gpu_memory_utilization=args.gpu_memory_utilization,
                 enforce_eager=args.enforce_eager, kvcache_block_size=args.kvcache_block_size,
                 num_kvcache_blocks=args.num_kvcache_blocks, dtype=args.dtype, seed=args.seed,
-                schedule=args.schedule, enable_prefix_caching=not args.no_prefix_caching)
+                schedule=args.schedule, enable_prefix_caching=not args.no_prefix_caching,
+                random_weights=args.random_weights)
 
 
 def cmd_generate(args) -> int:
@@ -50,6 +54,38 @@ def cmd_generate(args) -> int:
         for p, o in zip(prompts, outs):
             print(f"\nPrompt: {p!r}")
             print(f"Completion: {o['text']!r}" if o["text"] is not None else f"Completion ids: {o['token_ids']}")
+    return 0
+
+
+def cmd_throughput(args) -> int:
+    """The workload of the reference's bench.py (bench.py:9-28 there): num_seqs requests of
+    random token ids, prompt and output lengths uniform in [min, max], sampled at a
+    temperature with ignore_eos, after one short warm-up request; prints the reference's line
+    (generated tokens, seconds, tokens a second) and, with --json, the engine's own counts."""
+    import random
+    import time
+    from . import LLM, SamplingParams
+    rng = random.Random(args.workload_seed)
+    llm = LLM(args.model, **engine_kwargs(args))
+    vocab = llm.model.spec.vocab_size
+    top = min(vocab, args.max_token_id)
+    prompts = [[rng.randrange(top) for _ in range(rng.randint(args.min_input_len, args.max_input_len))]
+               for _ in range(args.num_seqs)]
+    params = [SamplingParams(temperature=args.temperature, ignore_eos=True,
+                             max_tokens=rng.randint(args.min_output_len, args.max_output_len))
+              for _ in range(args.num_seqs)]
+    llm.generate([[1, 2, 3, 4]], SamplingParams(temperature=args.temperature, max_tokens=8, ignore_eos=True),
+                 use_tqdm=False)
+    for k in llm.stats:
+        llm.stats[k] = 0 if isinstance(llm.stats[k], int) else 0.0
+    t0 = time.perf_counter()
+    llm.generate(prompts, params, use_tqdm=False)
+    dt = time.perf_counter() - t0
+    total = sum(p.max_tokens for p in params)
+    print(f"Total: {total}tok, Time: {dt:.2f}s, Throughput: {total / dt:.2f}tok/s")
+    if args.json:
+        print(json.dumps({"generated_tokens": total, "prompt_tokens": sum(len(p) for p in prompts), "seconds": dt,
+                          "tokens_per_second": total / dt, "num_seqs": args.num_seqs, **llm.stats}))
     return 0
 
 
@@ -74,6 +110,18 @@ def main(argv=None) -> int:
     g.add_argument("--ignore-eos", action="store_true")
     g.add_argument("--json", action="store_true", help="print the outputs as one JSON line")
     g.set_defaults(fn=cmd_generate)
+    t = sub.add_parser("throughput", help="requests of random tokens through generate (bench.py of the reference)")
+    add_engine_options(t)
+    t.add_argument("--num-seqs", type=int, default=256)
+    t.add_argument("--min-input-len", type=int, default=100)
+    t.add_argument("--max-input-len", type=int, default=1024)
+    t.add_argument("--min-output-len", type=int, default=100)
+    t.add_argument("--max-output-len", type=int, default=1024)
+    t.add_argument("--max-token-id", type=int, default=10000, help="prompt ids are drawn below this (and the vocabulary)")
+    t.add_argument("--temperature", type=float, default=0.6)
+    t.add_argument("--workload-seed", type=int, default=0)
+    t.add_argument("--json", action="store_true", help="also print the counts as one JSON line")
+    t.set_defaults(fn=cmd_throughput)
     r = sub.add_parser("random-model", help="write a model folder with seeded random weights")
     r.add_argument("--config", required=True, help="a config.json of the architecture")
     r.add_argument("--seed", type=int, default=0)

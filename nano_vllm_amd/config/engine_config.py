@@ -28,6 +28,7 @@ class EngineConfig:
     schedule: str = "prefill_first"         # the reference's policy, or "mixed"
     enable_prefix_caching: bool = True
     device: str = "cuda:0"
+    random_weights: Optional[int] = None    # a seed: the folder needs config.json only, weights are drawn on the device
 
     def __post_init__(self):
         if not os.path.isdir(self.model):                          # config.py:21

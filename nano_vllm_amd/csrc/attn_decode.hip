@@ -63,6 +63,23 @@ __device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf1
     for (int dt = 0; dt < DT; ++dt) vf[dt] = *reinterpret_cast<const bf16x8*>(pv + (int64_t)dt * 16 * vt);
 }
 
+// Keys per split: the longest split that still gives the GPU about 2048 waves when the longest
+// request of the step holds `longest` keys, at least 64 (32 where pages are tiny: a wave keeps its
+// split's block table entries in one register per lane, at most 62 pages).  The launcher and the
+// kernels share this function: a captured launch covers every length up to a bound, and the kernels
+// cut the splits for the step's real longest request, which they read from device memory.
+__host__ __device__ inline int nva_decode_split_len(int longest, int tokens, int kv_heads, int page_size) {
+    int len = 64;
+    for (int cand = 8192; cand >= 128; cand >>= 1)
+        if ((int64_t)tokens * kv_heads * ((longest + cand - 1) / cand) >= 2048) {
+            len = cand;
+            break;
+        }
+    const int cap = (62 * page_size) / DEC_CHUNK * DEC_CHUNK;
+    if (len > cap) len = cap;
+    return len < DEC_CHUNK ? DEC_CHUNK : len;
+}
+
 template <int D>
 __global__ void __launch_bounds__(NVA_WAVE)
 attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
@@ -71,7 +88,8 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
                    const int32_t* __restrict__ block_tables, int table_stride,
                    const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                    int num_q_heads, int num_kv_heads, int page_size, float scale, int window, int split_len,
-                   int num_splits, int32_t* error_flag) {
+                   int num_splits, const int32_t* __restrict__ longest, int32_t* error_flag) {
+    if (longest) split_len = nva_decode_split_len(*longest, (int)gridDim.z, num_kv_heads, page_size);
     constexpr int KP = D / 32;          // 16-byte pieces of a key row per lane = MFMAs per S tile
     constexpr int DT = D / 16;          // 16-channel tiles of the output
     const int split = blockIdx.x, kvh = blockIdx.y;
@@ -217,7 +235,9 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 __global__ void __launch_bounds__(MERGE_WAVES * NVA_WAVE)
 attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                          __bf16* __restrict__ out, int64_t out_stride, const int32_t* __restrict__ positions,
-                         int num_q_heads, int head_dim, int window, int split_len, int num_splits) {
+                         int num_q_heads, int num_kv_heads, int page_size, int head_dim, int window, int split_len,
+                         int num_splits, const int32_t* __restrict__ longest) {
+    if (longest) split_len = nva_decode_split_len(*longest, (int)gridDim.x, num_kv_heads, page_size);
     __shared__ float acc_s[MERGE_WAVES][4 * NVA_WAVE];
     __shared__ float l_s[MERGE_WAVES];
     const int64_t t = blockIdx.x;
@@ -271,14 +291,34 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
     }
 }
 
+// What a launch needs for `tokens` single tokens whose longest request holds at most `longest`
+// keys: the keys per split and the number of splits (the grid's width and the stride of the
+// partial results).  lengths_vary: the launch is captured and replayed for every length up to
+// `longest`; the number of splits then covers them all.
+NVA_EXPORT int nva_attn_decode_plan_bf16(int longest, int64_t tokens, int num_kv_heads, int page_size, int lengths_vary,
+                                    int* split_len, int* num_splits) {
+    if (longest <= 0 || tokens <= 0 || tokens > 65535 || num_kv_heads <= 0 || page_size <= 0 || !split_len || !num_splits)
+        return nva_fail("attn_decode_plan: bad arguments");
+    *split_len = nva_decode_split_len(longest, (int)tokens, num_kv_heads, page_size);
+    *num_splits = (longest + *split_len - 1) / *split_len;
+    if (lengths_vary)
+        for (int len = DEC_CHUNK; len < longest; len += DEC_CHUNK) {
+            const int s = nva_decode_split_len(len, (int)tokens, num_kv_heads, page_size);
+            if ((len + s - 1) / s > *num_splits) *num_splits = (len + s - 1) / s;
+        }
+    return 0;
+}
+
 // Returns 1 (and leaves a message) for shapes this kernel does not take; the caller then uses the
-// general kernel.  split_len must be a multiple of 32; num_splits = ceil(max kv length / split_len).
+// general kernel.  split_len and num_splits come from nva_attn_decode_plan.  longest: null, or a
+// device int32 with the keys of the step's longest request, from which the kernels then cut the
+// splits themselves (a captured launch, planned with lengths_vary).
 NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride, float* scratch,
                                     const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                     int table_stride, const int32_t* token_seq, const int32_t* positions,
                                     int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
-                                    float scale, int window, int split_len, int num_splits, int32_t* error_flag,
-                                    hipStream_t stream) {
+                                    float scale, int window, int split_len, int num_splits, const int32_t* longest,
+                                    int32_t* error_flag, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_decode: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
@@ -302,7 +342,7 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     hipLaunchKernelGGL(attn_decode_kernel<DD>, grid, dim3(NVA_WAVE), 0, stream, (const __bf16*)q, q_stride,       \
                        (__bf16*)out, out_stride, part_o, part_ml, (const __bf16*)k_cache, (const __bf16*)v_cache, \
                        block_tables, table_stride, token_seq, positions, num_q_heads, num_kv_heads, page_size,    \
-                       scale, window, split_len, num_splits, error_flag)
+                       scale, window, split_len, num_splits, longest, error_flag)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;
@@ -320,7 +360,8 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     if (num_splits > 1) {
         dim3 mgrid((unsigned)tokens, (unsigned)num_q_heads);
         hipLaunchKernelGGL(attn_decode_merge_kernel, mgrid, dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, (__bf16*)out,
-                           out_stride, positions, num_q_heads, head_dim, window, split_len, num_splits);
+                           out_stride, positions, num_q_heads, num_kv_heads, page_size, head_dim, window, split_len,
+                           num_splits, longest);
         rc = nva_check_launch("attn_decode_merge");
     }
     return rc;

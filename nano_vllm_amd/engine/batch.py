@@ -43,6 +43,7 @@ class StepBatch:
     kv_lens: torch.Tensor            # int32 [S] keys each request sees = start + its tokens
     seq_starts: torch.Tensor         # int32 [S] tokens each request had in the cache before
     state_slots: torch.Tensor        # int32 [S]
+    max_kv_dev: torch.Tensor         # int32 [1]: max(kv_lens), for kernels of a replayed launch
     logits_rows: Optional[torch.Tensor]   # int32 [R] flat token indices, in the caller's order
     prefill_tiles: Optional[torch.Tensor]  # int32 [tiles, 2]: (request, 32-row tile) of the portions, most keys first
     groups: List[GroupBatch]
@@ -52,17 +53,22 @@ class StepBatch:
     q_lens: List[int] = field(default_factory=list)
     starts: List[int] = field(default_factory=list)
     requests: List[Hashable] = field(default_factory=list)
+    lengths_vary: bool = False       # a captured launch: max_kv_len is a bound, max_kv_dev the step's value
 
 
 def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size: int, device,
-                table_width: Optional[int] = None, static: Optional[torch.Tensor] = None) -> StepBatch:
+                table_width: Optional[int] = None, static: Optional[torch.Tensor] = None,
+                pad_to: Optional[int] = None) -> StepBatch:
     """Orders the entries (single tokens first), checks them against the cache manager's
     block tables and uploads everything in one copy.
 
     table_width fixes the width of the block tables (else: the widest table of the batch).
     static, an int32 device tensor of the batch's flat size, receives the copy instead of a
     new tensor: with equal counts of tokens, requests and wanted places and a fixed table
-    width the layout is the same for every step, which is what a captured graph replays on."""
+    width the layout is the same for every step, which is what a captured graph replays on.
+    pad_to (decoded tokens only) fills the batch up to that many requests with copies of the
+    first entry that write nothing into the cache (slot -1): they read what the first request
+    reads, and their logits, which follow the real ones, are dropped by the caller."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
@@ -129,12 +135,27 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
                 raise ValueError(f"request {e.request!r}: position {where} has no page in group {g}")
             slot_maps[g].append(pages * page_size + pos % page_size)
     num_decode = len(one_ids)
+    pad = 0
+    if pad_to is not None and pad_to > S:
+        if num_decode != S:
+            raise ValueError("only a batch of decoded tokens can be padded")
+        pad = pad_to - S
+        one_ids += [one_ids[0]] * pad
+        one_pos += [one_pos[0]] * pad
+        for values in (kv_lens, starts, q_lens, state_slots):
+            values += [values[0]] * pad
+        cu += list(range(S + 1, S + pad + 1))
+        for g in range(num_groups):
+            one_slots[g] += [-1] * pad
+            tables[g] += [tables[g][0]] * pad
+        T, S, num_decode = T + pad, S + pad, num_decode + pad
     rows = []
     for i, e in enumerate(entries):
         for w in e.want:
             if not 0 <= w < len(e.tokens):
                 raise ValueError(f"request {e.request!r}: wanted place {w} is outside its {len(e.tokens)} tokens")
             rows.append(offsets[i] + w)
+    rows += list(range(T - pad, T))
 
     widths = [max(1, max(len(tb) for tb in tables[g])) for g in range(num_groups)]
     if table_width is not None:
@@ -142,7 +163,7 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
             raise ValueError(f"a block table of {max(widths)} pages exceeds the fixed width {table_width}")
         widths = [table_width] * num_groups
     tile_order = prefill_tile_order(q_lens, starts, num_decode)
-    scalars = cu + kv_lens + starts + state_slots + rows + tile_order
+    scalars = cu + kv_lens + starts + state_slots + [max(kv_lens)] + rows + tile_order
     if num_decode == S:                              # decoded tokens only: one list, one conversion
         flat: List[int] = one_ids + one_pos + list(range(S)) + scalars
         for g in range(num_groups):
@@ -180,7 +201,7 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
         return out
 
     b_ids, b_pos, b_seq = take(T), take(T), take(T)
-    b_cu, b_kv, b_starts, b_slots = take(S + 1), take(S), take(S), take(S)
+    b_cu, b_kv, b_starts, b_slots, b_max_kv = take(S + 1), take(S), take(S), take(S), take(1)
     b_rows = take(len(rows)) if rows else None
     b_tiles = take(len(tile_order)).view(-1, 2) if tile_order else None
     groups = []
@@ -191,6 +212,6 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
     return StepBatch(
         num_tokens=T, num_seqs=S, num_decode=num_decode, prefill_tiles=b_tiles,
         input_ids=b_ids, positions=b_pos, token_seq=b_seq, cu_seqlens_q=b_cu, kv_lens=b_kv,
-        seq_starts=b_starts, state_slots=b_slots, logits_rows=b_rows, groups=groups,
+        seq_starts=b_starts, state_slots=b_slots, max_kv_dev=b_max_kv, logits_rows=b_rows, groups=groups,
         max_q_len=max(q_lens), max_kv_len=max(kv_lens), q_lens=q_lens, starts=starts,
         requests=[entries[i].request for i in order])

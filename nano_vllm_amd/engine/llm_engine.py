@@ -32,7 +32,7 @@ class LLMEngine:
         if unknown:
             raise TypeError(f"unknown engine options {sorted(unknown)}; known: {sorted(EngineConfig.field_names())}")
         self.config = cfg = EngineConfig(model, **kwargs)
-        self.model = load_model(cfg.model, cfg.dtype, cfg.device, kernels)
+        self.model = load_model(cfg.model, cfg.dtype, cfg.device, kernels, random_weights=cfg.random_weights)
         spec = self.model.spec
         cfg.max_model_len = min(cfg.max_model_len, spec.max_position)           # config.py:25
         num_pages = cfg.num_kvcache_blocks

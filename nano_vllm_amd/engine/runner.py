@@ -19,6 +19,7 @@ from ..config.registry import architecture_of
 from ..kernels import HipKernels
 from ..parts.model import Model, torch_dtype
 from ..weights.loader import load_weights
+from ..weights.random_weights import fill_random_
 from .batch import StepBatch, StepEntry, build_batch
 
 
@@ -69,10 +70,10 @@ class ModelRunner:
     # ------------------------------------------------------------------ captured decode steps
     def enable_decode_graphs(self, max_batch: int, max_len: int) -> None:
         """Decode steps (one token per request, its logits wanted) of up to max_batch requests
-        and max_len cached tokens are captured as HIP graphs, one per batch size, at their
-        first occurrence, and replayed from then on.  Reference: capture_cudagraph and the
-        replay branch of run_model (nanovllm/engine/model_runner.py:195-212,222-257), which
-        pads to a few sizes instead."""
+        and max_len cached tokens are captured as HIP graphs, one per padded batch size, at
+        their first occurrence, and replayed from then on.  Reference: capture_cudagraph and
+        the replay branch of run_model (nanovllm/engine/model_runner.py:195-212,222-257),
+        which captures every size at start-up."""
         if self.state_runs:
             return          # a mixer with host-side state handling cannot be replayed blindly
         self._graph_max_batch = max_batch
@@ -87,18 +88,30 @@ class ModelRunner:
                 return False
         return True
 
+    @staticmethod
+    def graph_batch_size(n: int) -> int:
+        """The captured batch size that serves n requests: 1, 2, 4, 8, then multiples of 16
+        (the reference's buckets, nanovllm/engine/model_runner.py:226)."""
+        for b in (1, 2, 4, 8):
+            if n <= b:
+                return b
+        return (n + 15) // 16 * 16
+
     def _step_graph(self, entries) -> torch.Tensor:
         n = len(entries)
+        size_b = self.graph_batch_size(n)
         vocab = self.model.spec.vocab_size
-        g = self._graphs.get(n)
+        g = self._graphs.get(size_b)
         if g is None:
-            # the flat layout of n single tokens with every logit wanted and tables of fixed width
+            # the flat layout of size_b single tokens with every logit wanted and tables of fixed width
             num_groups = len(self.groups)
-            size = 3 * n + (n + 1) + 3 * n + n + num_groups * (n + n * self._graph_table_width)
+            b = size_b
+            size = 3 * b + (b + 1) + 3 * b + 1 + b + num_groups * (b + b * self._graph_table_width)
             static = torch.zeros(size, dtype=torch.int32, device=self.device)
             batch = build_batch(entries, self.cache, self.page_size, vocab, self.device,
-                                table_width=self._graph_table_width, static=static)
+                                table_width=self._graph_table_width, static=static, pad_to=size_b)
             batch.max_kv_len = self._graph_max_len        # launch shapes must cover every later step
+            batch.lengths_vary = True
             side = torch.cuda.Stream(self.device)
             side.wait_stream(torch.cuda.current_stream(self.device))
             with torch.cuda.stream(side):                 # what is set up lazily is set up outside the capture
@@ -110,16 +123,18 @@ class ModelRunner:
             with torch.cuda.graph(graph):
                 logits = self.model.logits(self.model.forward(batch, self.layer_caches), batch.logits_rows)
             g = (graph, static, logits)
-            self._graphs[n] = g
+            self._graphs[size_b] = g
         graph, static, logits = g
         build_batch(entries, self.cache, self.page_size, vocab, self.device,
-                    table_width=self._graph_table_width, static=static)
+                    table_width=self._graph_table_width, static=static, pad_to=size_b)
         graph.replay()
-        return logits
+        return logits[:n]
 
 
-def load_model(folder: str, dtype: Optional[str] = None, device="cuda:0", kernels=None, quiet: bool = False) -> Model:
-    """config.json -> architecture -> ModelSpec -> Model, then the weights of the folder."""
+def load_model(folder: str, dtype: Optional[str] = None, device="cuda:0", kernels=None, quiet: bool = False,
+               random_weights: Optional[int] = None) -> Model:
+    """config.json -> architecture -> ModelSpec -> Model, then the weights of the folder, or,
+    with a seed in random_weights, random weights drawn on the device."""
     config_json = read_config_json(folder)
     arch = architecture_of(config_json)
     config = arch.parse_config(config_json)
@@ -128,5 +143,8 @@ def load_model(folder: str, dtype: Optional[str] = None, device="cuda:0", kernel
     if kernels is None:
         kernels = HipKernels(device, tdtype, quiet=quiet)        # raises without a GPU or the compiled kernels
     model = Model(spec, kernels, device, tdtype)
-    load_weights(model, folder)
+    if random_weights is None:
+        load_weights(model, folder)
+    else:
+        fill_random_(model, random_weights)
     return model

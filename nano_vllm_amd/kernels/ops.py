@@ -491,15 +491,18 @@ class HipKernels:
 
     def _attention_decode(self, q, qs, out, os_, k_cache, v_cache, tables, batch, n, num_heads, num_kv_heads,
                           head_dim, page_size, scale, window):
-        max_kv = batch.max_kv_len
-        split_len = 64
-        for cand in (8192, 4096, 2048, 1024, 512, 256, 128):       # the longest split that still fills the GPU
-            if n * num_kv_heads * ((max_kv + cand - 1) // cand) >= 2048:
-                split_len = cand
-                break
-        # a wave keeps its split's block table entries in one register per lane: at most 62 pages
-        split_len = max(32, min(split_len, (62 * page_size) // 32 * 32))
-        num_splits = (max_kv + split_len - 1) // split_len
+        # keys per split and number of splits: the kernels' own rule (one place, in the library).  A
+        # batch that a captured graph replays covers every length up to its bound, and the kernels read
+        # the step's longest request from the batch's device copy.
+        vary = bool(getattr(batch, "lengths_vary", False))
+        longest = getattr(batch, "max_kv_dev", None) if vary else None
+        if vary and (longest is None or n > 65535):
+            raise KernelError("attention: a batch whose lengths vary needs max_kv_dev and at most 65535 tokens")
+        split_len, num_splits = ctypes.c_int(0), ctypes.c_int(0)
+        library.call("attn_decode", "bf16", "nva_attn_decode_plan", c_i32(batch.max_kv_len), c_i64(min(n, 65535)),
+                     c_i32(num_kv_heads), c_i32(page_size), c_i32(1 if vary else 0), ctypes.byref(split_len),
+                     ctypes.byref(num_splits))
+        split_len, num_splits = split_len.value, num_splits.value
         scratch = None
         if num_splits > 1:
             scratch = torch.empty(n * num_heads * num_splits * (head_dim + 2), dtype=torch.float32, device=q.device)
@@ -509,7 +512,7 @@ class HipKernels:
                          _p(scratch), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          _p(batch.token_seq[t0:t1]), _p(batch.positions[t0:t1]), c_i64(t1 - t0), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         c_i32(split_len), c_i32(num_splits), _p(self.fault_flag), self._stream())
+                         c_i32(split_len), c_i32(num_splits), _p(longest), _p(self.fault_flag), self._stream())
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:

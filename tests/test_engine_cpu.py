@@ -75,6 +75,31 @@ def test_logits_come_back_in_the_callers_order():
     assert H.rel_err(out, want) < TOL
 
 
+def test_a_padded_batch_of_decoded_tokens_reads_what_the_first_request_reads():
+    """The captured decode graphs run a few fixed batch sizes: the rows beyond the real requests
+    are copies of the first entry that write nothing, and the real rows are not changed by them."""
+    from nano_vllm_amd.engine.batch import build_batch
+    r = _runner("a", 16)
+    toks = {rid: H.random_tokens(256, 9, s) for s, rid in enumerate("pqr")}
+    for rid, t in toks.items():
+        r.cache.admit(rid)
+        r.cache.reserve(rid, 9)
+        r.step([StepEntry(rid, t[:8], 0, [])])
+    entries = [StepEntry(rid, t[8:], 8, [0]) for rid, t in toks.items()]
+    b = build_batch(entries, r.cache, r.page_size, 256, "cpu", table_width=5, pad_to=4)
+    assert (b.num_seqs, b.num_tokens, b.num_decode) == (4, 4, 4)
+    assert b.input_ids.tolist() == [toks["p"][8], toks["q"][8], toks["r"][8], toks["p"][8]]
+    assert b.positions.tolist() == [8, 8, 8, 8] and b.logits_rows.tolist() == [0, 1, 2, 3]
+    assert b.groups[0].slot_mapping.tolist()[3] == -1 and b.groups[0].slot_mapping.tolist()[0] >= 0
+    assert b.groups[0].block_tables[3].tolist() == b.groups[0].block_tables[0].tolist()
+    assert b.groups[0].block_tables.shape == (4, 5)
+    padded = r.model.logits(r.model.forward(b, r.layer_caches), b.logits_rows)
+    plain_rows = r.step(entries)
+    assert torch.equal(padded[:3], plain_rows) and torch.equal(padded[3], padded[0])
+    with pytest.raises(ValueError, match="decoded"):
+        build_batch([StepEntry("p", toks["p"][7:], 7, [])], r.cache, r.page_size, 256, "cpu", pad_to=2)
+
+
 def _llm(name, **kw):
     c = H.CONFIGS[name]
     opts = dict(kernels=TorchKernels(), device="cpu", dtype="float32", kvcache_block_size=c["page"],

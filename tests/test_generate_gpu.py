@@ -92,3 +92,23 @@ def test_command_line_generates(tmp_path):
     outs = json.loads(proc.stdout.strip().split("\n")[-1])
     cfg, w = plain.read_folder(H.model_folder("b", "float32"))
     assert [o["token_ids"] for o in outs] == [plain.greedy_generate(w, cfg, p, 4) for p in ([5, 6, 7], [9, 8])]
+
+
+def test_throughput_command_with_weights_drawn_on_the_device(tmp_path, capsys):
+    """The reference's bench.py workload in small: requests of random ids through generate, with
+    the weights drawn from a seed (the folder holds config.json only), padded decode graphs and
+    so few pages that requests wait and are preempted."""
+    from nano_vllm_amd.cli import main
+    folder = tmp_path / "config_only"
+    folder.mkdir()
+    cj = H.CONFIGS["c"]["cfg"].to_dict()
+    (folder / "config.json").write_text(json.dumps(cj))
+    rc = main(["throughput", "--model", str(folder), "--random-weights", "4", "--num-seqs", "11", "--min-input-len", "5",
+               "--max-input-len", "60", "--min-output-len", "4", "--max-output-len", "40", "--max-token-id", "500",
+               "--kvcache-block-size", "16", "--num-kvcache-blocks", "24", "--max-num-seqs", "6",
+               "--max-num-batched-tokens", "64", "--max-model-len", "128", "--json"])
+    assert rc == 0
+    lines = capsys.readouterr().out.strip().split("\n")
+    assert lines[-2].startswith("Total: ") and "Throughput: " in lines[-2]
+    stats = json.loads(lines[-1])
+    assert stats["num_seqs"] == 11 and stats["decode_tokens"] > 0 and stats["prefill_tokens"] >= stats["prompt_tokens"]
