@@ -7,6 +7,7 @@ from __future__ import annotations
 
 from typing import List, Sequence
 
+import numpy as np
 import torch
 
 _M64 = (1 << 64) - 1
@@ -25,18 +26,43 @@ def noise_key(seed: int, request: int, position: int) -> int:
     return key - (1 << 64) if key >= (1 << 63) else key
 
 
+def noise_keys(seeds: Sequence[int], requests: Sequence[int], positions: Sequence[int]) -> "np.ndarray":
+    """noise_key of many draws at once, as int64 (the same integers, computed modulo 2^64)."""
+    def mix(z):
+        z = z + np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+    as_u64 = lambda values: np.array([v & _M64 for v in values], dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        return mix(mix(mix(as_u64(seeds)) ^ as_u64(requests)) ^ as_u64(positions)).view(np.int64)
+
+
 class Sampler:
+    """Holds the device copies of what rarely changes from step to step (the temperatures of
+    the batch; the unused keys of a batch that is all greedy), so that a decode step of the
+    same requests uploads nothing, or only its keys."""
+
     def __init__(self, kernels, device):
         self.kernels = kernels
         self.device = device
+        self._temps = None            # (tuple of temperatures, device tensor)
+        self._zero_keys = None
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
                requests: Sequence[int], positions: Sequence[int]) -> List[int]:
         """One token per row of logits.  positions: the position the new token will take."""
         n = logits.shape[0]
-        keys = [noise_key(s, r, p) for s, r, p in zip(seeds, requests, positions)]
-        temps = torch.tensor(list(temperatures), dtype=torch.float32).to(self.device)
-        keys_t = torch.tensor(keys, dtype=torch.int64).to(self.device)
-        assert temps.shape[0] == n and keys_t.shape[0] == n
-        ids = self.kernels.sample(logits, temps, keys_t)
+        temps = tuple(float(t) for t in temperatures)
+        assert len(temps) == n and len(seeds) == n and len(requests) == n and len(positions) == n
+        if self._temps is None or self._temps[0] != temps:
+            self._temps = (temps, torch.tensor(temps, dtype=torch.float32).to(self.device))
+        if any(t > 0.0 for t in temps):
+            keys_t = torch.from_numpy(noise_keys(seeds, requests, positions)).to(self.device)
+        else:
+            if self._zero_keys is None or self._zero_keys.shape[0] < n:
+                self._zero_keys = torch.zeros(max(n, 64), dtype=torch.int64, device=self.device)
+            keys_t = self._zero_keys[:n]
+        ids = self.kernels.sample(logits, self._temps[1], keys_t)
         return ids.tolist()
