@@ -1,4 +1,5 @@
-// Next-token choice from float logits, one block per row.
+// Next-token choice from float logits: one block per chunk of 8192 entries of a row, then one
+// wave per row over the chunks' results.
 //
 // temperature == 0: the argmax of the logits, the lowest index on ties.
 // temperature  > 0: the reference draws argmax(softmax(l / T) / E) with E ~ Exp(1) i.i.d. per
@@ -18,59 +19,33 @@ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
     return z ^ (z >> 31);
 }
 
-#define SAMPLE_THREADS 1024
+#define SAMPLE_THREADS 256
+#define SAMPLE_CHUNK 8192         // entries of a row per workgroup
 
-__device__ __forceinline__ void take(double s, int i, double& best, int& best_idx) {
-    // a NaN score never wins; a row of only NaN yields index 0
-    if (s == s && (best_idx == 0x7fffffff || s > best || (s == best && i < best_idx))) {
-        best = s;
-        best_idx = i;
-    }
+__device__ __forceinline__ bool better(double s, int i, double best, int best_idx) {
+    // a NaN score never wins (its index stays 0x7fffffff); the lowest index wins a tie
+    return i != 0x7fffffff && (best_idx == 0x7fffffff || s > best || (s == best && i < best_idx));
 }
 
-__global__ void __launch_bounds__(SAMPLE_THREADS)
-sample_kernel(const float* __restrict__ logits, int64_t row_stride, int vocab,
-              const float* __restrict__ temperatures, const uint64_t* __restrict__ keys,
-              int32_t* __restrict__ out) {
+__device__ __forceinline__ double score(float logit, float temp, uint64_t key, int entry) {
+    double s = (double)logit;
+    if (temp > 0.f) {
+        const uint64_t bits = mix64(key ^ (uint64_t)entry);
+        const double u = ((double)(bits >> 40) + 0.5) * (1.0 / 16777216.0);
+        s = s / (double)temp - log(-log(u));
+    }
+    return s;
+}
+
+// The best entry of a block's threads: within the waves, then across them (thread 0 holds it).
+__device__ __forceinline__ void block_best(double& best, int& best_idx) {
     __shared__ double best_s[SAMPLE_THREADS / NVA_WAVE];
     __shared__ int best_i[SAMPLE_THREADS / NVA_WAVE];
-    const int64_t row = blockIdx.x;
-    const float* l = logits + row * row_stride;
-    const float temp = temperatures ? temperatures[row] : 0.f;
-    const uint64_t key = keys ? keys[row] : 0;
-    double best = -INFINITY;
-    int best_idx = 0x7fffffff;
-    const bool vec = (row_stride % 4 == 0) && ((uintptr_t)logits % 16 == 0);
-    const int vec_end = vec ? (vocab & ~3) : 0;
-    for (int i = threadIdx.x * 4; i < vec_end; i += blockDim.x * 4) {
-        const float4 v4 = *reinterpret_cast<const float4*>(l + i);
-        const float v[4] = {v4.x, v4.y, v4.z, v4.w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            double s = (double)v[e];
-            if (temp > 0.f) {
-                const uint64_t bits = mix64(key ^ (uint64_t)(i + e));
-                const double u = ((double)(bits >> 40) + 0.5) * (1.0 / 16777216.0);
-                s = s / (double)temp - log(-log(u));
-            }
-            take(s, i + e, best, best_idx);
-        }
-    }
-    for (int i = vec_end + threadIdx.x; i < vocab; i += blockDim.x) {
-        double s = (double)l[i];
-        if (temp > 0.f) {
-            const uint64_t bits = mix64(key ^ (uint64_t)i);
-            const double u = ((double)(bits >> 40) + 0.5) * (1.0 / 16777216.0);
-            s = s / (double)temp - log(-log(u));
-        }
-        take(s, i, best, best_idx);
-    }
-    // within the wave, then across the waves
 #pragma unroll
     for (int off = NVA_WAVE / 2; off > 0; off >>= 1) {
         const double os = __shfl_xor(best, off, NVA_WAVE);
         const int oi = __shfl_xor(best_idx, off, NVA_WAVE);
-        if (oi != 0x7fffffff && (best_idx == 0x7fffffff || os > best || (os == best && oi < best_idx))) {
+        if (better(os, oi, best, best_idx)) {
             best = os;
             best_idx = oi;
         }
@@ -81,26 +56,103 @@ sample_kernel(const float* __restrict__ logits, int64_t row_stride, int vocab,
         best_i[wave] = best_idx;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int w = 1; w < blockDim.x / NVA_WAVE; ++w) {
-            const double os = best_s[w];
-            const int oi = best_i[w];
-            if (oi != 0x7fffffff && (best_idx == 0x7fffffff || os > best || (os == best && oi < best_idx))) {
-                best = os;
-                best_idx = oi;
+    if (threadIdx.x == 0)
+        for (int w = 1; w < (int)blockDim.x / NVA_WAVE; ++w)
+            if (better(best_s[w], best_i[w], best, best_idx)) {
+                best = best_s[w];
+                best_idx = best_i[w];
+            }
+}
+
+// First pass: the best entry of one chunk of one row -> part_s / part_i [rows][chunks].
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_chunk_kernel(const float* __restrict__ logits, int64_t row_stride, int vocab,
+                    const float* __restrict__ temperatures, const uint64_t* __restrict__ keys,
+                    double* __restrict__ part_s, int32_t* __restrict__ part_i) {
+    const int64_t row = blockIdx.y;
+    const int chunk = blockIdx.x, chunks = gridDim.x;
+    const float* l = logits + row * row_stride;
+    const float temp = temperatures ? temperatures[row] : 0.f;
+    const uint64_t key = keys ? keys[row] : 0;
+    const int begin = chunk * SAMPLE_CHUNK, end = min(vocab, begin + SAMPLE_CHUNK);
+    double best = -INFINITY;
+    int best_idx = 0x7fffffff;
+    const bool vec = (row_stride % 4 == 0) && ((uintptr_t)logits % 16 == 0);
+    const int vec_end = vec ? begin + ((end - begin) & ~3) : begin;
+    for (int i = begin + threadIdx.x * 4; i < vec_end; i += SAMPLE_THREADS * 4) {
+        const float4 v4 = *reinterpret_cast<const float4*>(l + i);
+        const float v[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const double s = score(v[e], temp, key, i + e);
+            if (s == s && better(s, i + e, best, best_idx)) {
+                best = s;
+                best_idx = i + e;
             }
         }
-        out[row] = best_idx == 0x7fffffff ? 0 : best_idx;
+    }
+    for (int i = vec_end + threadIdx.x; i < end; i += SAMPLE_THREADS) {
+        const double s = score(l[i], temp, key, i);
+        if (s == s && better(s, i, best, best_idx)) {
+            best = s;
+            best_idx = i;
+        }
+    }
+    block_best(best, best_idx);
+    if (threadIdx.x == 0) {
+        part_s[row * chunks + chunk] = best;
+        part_i[row * chunks + chunk] = best_idx;
     }
 }
 
+// Second pass: the best of a row's chunks; a row of only NaN yields index 0.
+__global__ void __launch_bounds__(NVA_WAVE)
+sample_merge_kernel(const double* __restrict__ part_s, const int32_t* __restrict__ part_i, int chunks,
+                    int32_t* __restrict__ out) {
+    const int64_t row = blockIdx.x;
+    double best = -INFINITY;
+    int best_idx = 0x7fffffff;
+    for (int c = threadIdx.x; c < chunks; c += NVA_WAVE) {
+        const double s = part_s[row * chunks + c];
+        const int i = part_i[row * chunks + c];
+        if (better(s, i, best, best_idx)) {
+            best = s;
+            best_idx = i;
+        }
+    }
+#pragma unroll
+    for (int off = NVA_WAVE / 2; off > 0; off >>= 1) {
+        const double os = __shfl_xor(best, off, NVA_WAVE);
+        const int oi = __shfl_xor(best_idx, off, NVA_WAVE);
+        if (better(os, oi, best, best_idx)) {
+            best = os;
+            best_idx = oi;
+        }
+    }
+    if (threadIdx.x == 0) out[row] = best_idx == 0x7fffffff ? 0 : best_idx;
+}
+
+// scratch: rows * ceil(vocab / 8192) * 12 bytes, 8-byte aligned (nva_sample_scratch_bytes).
+NVA_EXPORT int64_t nva_sample_scratch_bytes(int64_t rows, int vocab) {
+    const int64_t chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+    return rows * chunks * 12;
+}
+
 NVA_EXPORT int nva_sample(const float* logits, int64_t row_stride, int64_t rows, int vocab,
-                          const float* temperatures, const uint64_t* keys, int32_t* out, hipStream_t stream) {
+                          const float* temperatures, const uint64_t* keys, int32_t* out, void* scratch,
+                          hipStream_t stream) {
     if (rows == 0) return 0;
-    if (rows < 0 || rows > 0x7fffffff || vocab <= 0) return nva_fail("sample: bad shape rows=%lld vocab=%d", (long long)rows, vocab);
-    hipLaunchKernelGGL(sample_kernel, dim3((unsigned)rows), dim3(SAMPLE_THREADS), 0, stream, logits, row_stride, vocab,
-                       temperatures, keys, out);
-    return nva_check_launch("sample");
+    if (rows < 0 || rows > 65535 || vocab <= 0) return nva_fail("sample: bad shape rows=%lld vocab=%d", (long long)rows, vocab);
+    if (!scratch || !nva_aligned(scratch, 8)) return nva_fail("sample: needs 8-byte aligned scratch memory");
+    const int chunks = (vocab + SAMPLE_CHUNK - 1) / SAMPLE_CHUNK;
+    double* part_s = (double*)scratch;
+    int32_t* part_i = (int32_t*)(part_s + rows * chunks);
+    hipLaunchKernelGGL(sample_chunk_kernel, dim3((unsigned)chunks, (unsigned)rows), dim3(SAMPLE_THREADS), 0, stream, logits,
+                       row_stride, vocab, temperatures, keys, part_s, part_i);
+    int rc = nva_check_launch("sample_chunk");
+    if (rc) return rc;
+    hipLaunchKernelGGL(sample_merge_kernel, dim3((unsigned)rows), dim3(NVA_WAVE), 0, stream, part_s, part_i, chunks, out);
+    return nva_check_launch("sample_merge");
 }
 
 NVA_DEFINE_LAST_ERROR(nva_sample)

@@ -525,7 +525,12 @@ class HipKernels:
             raise KernelError("sample: temperatures must be float32 [rows]")
         if keys.dtype != torch.int64 or keys.shape != (rows,) or not keys.is_contiguous():
             raise KernelError("sample: keys must be int64 [rows]")
+        if rows > 65535:
+            raise KernelError("sample: at most 65535 rows a call")
         out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        need = library.load("sample", None).nva_sample_scratch_bytes
+        need.restype = ctypes.c_int64
+        scratch = torch.empty((int(need(c_i64(rows), c_i32(vocab))) + 7) // 8, dtype=torch.float64, device=logits.device)
         library.call("sample", None, "nva_sample", _p(logits), c_i64(stride), c_i64(rows), c_i32(vocab),
-                     _p(temperatures), _p(keys), _p(out), self._stream())
+                     _p(temperatures), _p(keys), _p(out), _p(scratch), self._stream())
         return out

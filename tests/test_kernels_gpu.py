@@ -419,6 +419,30 @@ def test_sampling_matches_the_plain_draw(hip):
     assert got == want and got[0] == 17
 
 
+def test_sampling_over_a_vocabulary_of_several_chunks(hip):
+    """A row is cut into chunks of 8192 entries for the first pass: ties across chunks, a maximum
+    at a chunk's edge, rows of a wider tensor (a stride that is no multiple of four), NaN entries."""
+    from nano_vllm_amd.sampling.sampler import noise_key
+    k = hip[torch.float32]
+    V, R = 20011, 5
+    wide = _rand((R, V + 3), torch.float32, 26, 2.0)
+    logits = wide[:, 1:V + 1]                                       # stride V + 3, first entry unaligned
+    logits[0, 8191] = logits[0, 8192] = logits[0, 20010] = 40.0     # a tie across chunks: the lowest index
+    logits[1, 16384] = 40.0                                         # first entry of the last chunk
+    logits[2, V - 1] = 40.0                                         # the very last entry
+    logits[3, :] = float("nan")                                     # nothing wins: index 0
+    logits[4, 5] = float("nan")
+    temps = torch.tensor([0.0, 0.0, 0.0, 0.0, 0.9], device=DEV)
+    keys = torch.tensor([noise_key(3, r, 7) for r in range(R)], dtype=torch.int64, device=DEV)
+    got = k.sample(logits, temps, keys).tolist()
+    assert got[:4] == [8191, 16384, V - 1, 0]
+    row = logits[4].cpu().clone()
+    row[5] = -1e30                                                  # the plain draw has no rule for NaN
+    assert got[4] == plain.sample(row, 0.9, seed=3, request=4, position=7)
+    aligned = logits.contiguous()
+    assert k.sample(aligned, temps, keys).tolist() == got
+
+
 def test_sampling_frequencies_follow_the_softmax(hip):
     from nano_vllm_amd.sampling.sampler import noise_key
     l = torch.tensor([1.0, 0.0, -1.0, 0.5, -2.0, 0.2, -0.3])
