@@ -36,6 +36,8 @@ def parse_args():
     ap.add_argument("--page-size", type=int, default=256)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes")
     ap.add_argument("--eager", action="store_true", help="no captured decode graph")
+    ap.add_argument("--burst", type=int, default=8,
+                    help="decode steps in a row without the host in between (the engine's decode_burst; 1: one)")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
 
@@ -101,22 +103,28 @@ def main():
         pos = start
         temps, seeds, reqs = [0.0] * batch, [0] * batch, list(range(batch))
 
-        def one_step():
+        def some_steps(count):
+            """`count` decode steps: through the host one by one, or as bursts on the device."""
             nonlocal tokens, pos
-            entries = []
-            for rid, tok in zip(ids, tokens):
-                runner.cache.reserve(rid, pos + 1)
-                entries.append(StepEntry(rid, [tok], pos, [0]))
-            logits = runner.step(entries)
-            tokens = sampler.sample(logits, temps, seeds, reqs, [pos + 1] * batch)
-            pos += 1
+            burst = 1 if args.eager else max(1, args.burst)
+            while count > 0:
+                n = min(burst, count)
+                entries = []
+                for rid, tok in zip(ids, tokens):
+                    runner.cache.reserve(rid, pos + n)
+                    entries.append(StepEntry(rid, [tok], pos, [0]))
+                if n == 1:
+                    logits = runner.step(entries)
+                    tokens = sampler.sample(logits, temps, seeds, reqs, [pos + 1] * batch)
+                else:
+                    tokens = runner.decode_burst(entries, n, sampler, temps, seeds, reqs)[-1]
+                pos += n
+                count -= n
 
-        for _ in range(warmup):
-            one_step()
+        some_steps(warmup)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            one_step()
+        some_steps(steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         assert pos == args.context
@@ -168,7 +176,8 @@ def main():
                    "parallelism": "single GPU", "layers": L, "layers_of_shape": full_layers, "hidden_size": H,
                    "num_attention_heads": Hq, "num_key_value_heads": Hkv, "head_dim": D, "intermediate_size": I,
                    "vocab_size": V, "kv_page_size": page, "prefill_tokens": T, "rope_theta": cfg.rope_theta,
-                   "rms_norm_eps": cfg.rms_norm_eps, "decode_graph": bool(not args.eager and hasattr(runner, "enable_decode_graphs"))},
+                   "rms_norm_eps": cfg.rms_norm_eps, "decode_graph": bool(not args.eager and hasattr(runner, "enable_decode_graphs")),
+                   "decode_burst": 1 if args.eager else max(1, args.burst)},
         "prefill": {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
                     "frac": round(prefill_flops / pre_s / PEAK_FLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

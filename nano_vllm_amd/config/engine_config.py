@@ -28,6 +28,7 @@ class EngineConfig:
     schedule: str = "prefill_first"         # the reference's policy, or "mixed"
     enable_prefix_caching: bool = True
     device: str = "cuda:0"
+    decode_burst: int = 4                   # decode steps in a row without the host, while no request waits (1: never)
     random_weights: Optional[int] = None    # a seed: the folder needs config.json only, weights are drawn on the device
 
     def __post_init__(self):
@@ -41,6 +42,8 @@ class EngineConfig:
             raise ConfigError("max_num_batched_tokens, max_num_seqs and max_model_len must be positive")
         if not (0 < self.gpu_memory_utilization <= 1):
             raise ConfigError("gpu_memory_utilization must lie in (0, 1]")
+        if self.decode_burst < 1:
+            raise ConfigError("decode_burst must be at least 1")
         if self.schedule not in ("prefill_first", "mixed"):
             raise ConfigError(f"schedule must be 'prefill_first' or 'mixed', got {self.schedule!r}")
         if self.dtype is not None:

@@ -155,4 +155,64 @@ NVA_EXPORT int nva_sample(const float* logits, int64_t row_stride, int64_t rows,
     return nva_check_launch("sample_merge");
 }
 
+// After a decode step whose tokens were just sampled: the step's own metadata, in place, becomes
+// that of the next decode step of the same requests (the reference rebuilds it on the host,
+// nanovllm/engine/model_runner.py:166-188; here several steps run without the host in between).
+// Request i < n_real takes its sampled token at the next position, whose slot comes from its block
+// tables (the page must be there already); rows n_real.. are padding: copies of request 0 that
+// write nothing.  out_row receives the sampled tokens.
+#define ADVANCE_MAX_GROUPS 4
+struct AdvanceGroups {
+    int32_t* slots[ADVANCE_MAX_GROUPS];
+    const int32_t* tables[ADVANCE_MAX_GROUPS];
+    int width[ADVANCE_MAX_GROUPS];
+};
+
+__global__ void advance_decode_kernel(int32_t* __restrict__ input_ids, int32_t* __restrict__ positions,
+                                      int32_t* __restrict__ kv_lens, int32_t* __restrict__ starts,
+                                      int32_t* __restrict__ max_kv, const int32_t* __restrict__ sampled,
+                                      int32_t* __restrict__ out_row, int n_real, int n_total, int page_size,
+                                      AdvanceGroups groups, int num_groups, int32_t* error_flag) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_total) return;
+    const int tok = sampled[i < n_real ? i : 0];
+    if (i < n_real) out_row[i] = tok;
+    const int pos = positions[i] + 1;
+    positions[i] = pos;
+    kv_lens[i] = pos + 1;
+    starts[i] = pos;
+    input_ids[i] = tok;
+    for (int g = 0; g < num_groups; ++g) {
+        int slot = -1;
+        if (i < n_real) {
+            const int page = pos / page_size < groups.width[g] ? groups.tables[g][(int64_t)i * groups.width[g] + pos / page_size] : -1;
+            if (page < 0) {
+                if (error_flag) atomicOr(error_flag, 2);
+            } else {
+                slot = page * page_size + pos % page_size;
+            }
+        }
+        groups.slots[g][i] = slot;
+    }
+    if (i == 0) max_kv[0] += 1;
+}
+
+NVA_EXPORT int nva_advance_decode(int32_t* input_ids, int32_t* positions, int32_t* kv_lens, int32_t* starts,
+                                  int32_t* max_kv, const int32_t* sampled, int32_t* out_row, int n_real, int n_total,
+                                  int page_size, int num_groups, int32_t* const* slots, const int32_t* const* tables,
+                                  const int* widths, int32_t* error_flag, hipStream_t stream) {
+    if (n_real <= 0 || n_total < n_real || page_size <= 0 || num_groups < 0 || num_groups > ADVANCE_MAX_GROUPS)
+        return nva_fail("advance_decode: bad sizes (%d of %d requests, %d cache groups)", n_real, n_total, num_groups);
+    AdvanceGroups groups;
+    for (int g = 0; g < num_groups; ++g) {
+        groups.slots[g] = slots[g];
+        groups.tables[g] = tables[g];
+        groups.width[g] = widths[g];
+    }
+    hipLaunchKernelGGL(advance_decode_kernel, dim3((unsigned)((n_total + 255) / 256)), dim3(256), 0, stream, input_ids,
+                       positions, kv_lens, starts, max_kv, sampled, out_row, n_real, n_total, page_size, groups, num_groups,
+                       error_flag);
+    return nva_check_launch("advance_decode");
+}
+
 NVA_DEFINE_LAST_ERROR(nva_sample)

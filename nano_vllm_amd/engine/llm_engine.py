@@ -127,17 +127,30 @@ class LLMEngine:
                 entries.append(StepEntry(seq.seq_id, seq.token_ids[start:start + n], start, [n - 1] if last else []))
                 if last:
                     sampled.append(seq)
-            logits = self.runner.step(entries)
-            tokens = {}
-            if sampled:
-                ids = self.sampler.sample(
-                    logits, [s.temperature for s in sampled],
-                    [self.config.seed if s.seed is None else s.seed for s in sampled],
-                    [s.seq_id for s in sampled], [s.num_tokens for s in sampled])
-                tokens = {s.seq_id: t for s, t in zip(sampled, ids)}
-            elif self.model.device.type == "cuda":
-                torch.cuda.synchronize(self.model.device)
-            self.scheduler.postprocess(seqs, [tokens.get(s.seq_id, -1) for s in seqs])
+            burst = self._burst_steps(seqs, entries, is_prefill)
+            if burst > 1:
+                rows = self.runner.decode_burst(
+                    entries, burst, self.sampler, [s.temperature for s in seqs],
+                    [self.config.seed if s.seed is None else s.seed for s in seqs], [s.seq_id for s in seqs])
+                for row in rows:                 # as after `burst` single steps; what follows a request's end is dropped
+                    live = [(s, t) for s, t in zip(seqs, row) if not s.is_finished]
+                    for s, _ in live:
+                        s.num_scheduled_tokens = 1
+                    self.scheduler.postprocess([s for s, _ in live], [t for _, t in live])
+                    self.stats["decode_tokens"] += len(live)
+                self.stats["decode_tokens"] -= len(seqs)            # the first row is counted below
+            else:
+                logits = self.runner.step(entries)
+                tokens = {}
+                if sampled:
+                    ids = self.sampler.sample(
+                        logits, [s.temperature for s in sampled],
+                        [self.config.seed if s.seed is None else s.seed for s in sampled],
+                        [s.seq_id for s in sampled], [s.num_tokens for s in sampled])
+                    tokens = {s.seq_id: t for s, t in zip(sampled, ids)}
+                elif self.model.device.type == "cuda":
+                    torch.cuda.synchronize(self.model.device)
+                self.scheduler.postprocess(seqs, [tokens.get(s.seq_id, -1) for s in seqs])
             num_tokens = sum(len(e.tokens) for e in entries) if is_prefill else -len(seqs)
             dt = perf_counter() - t0
             kind = "prefill" if is_prefill else "decode"
@@ -148,6 +161,30 @@ class LLMEngine:
         self.scheduler.just_finished = []
         outputs = [(s.seq_id, s.completion_token_ids) for s in finished]
         return outputs, num_tokens
+
+    def _burst_steps(self, seqs, entries, is_prefill) -> int:
+        """How many decode steps to run in a row without the host: more than one only while
+        no request waits, every request of the step decodes, the captured steps take the batch,
+        and pages for all the steps can be reserved; never past a request's last token."""
+        want = self.config.decode_burst
+        if want <= 1 or is_prefill or self.scheduler.waiting or not seqs:
+            return 1
+        runner = self.runner
+        if not (getattr(runner, "_graph_max_batch", 0) and runner._graph_takes(entries)):
+            return 1
+        for s in seqs:
+            if s.num_cached_tokens + 1 != s.num_tokens:
+                return 1
+            want = min(want, s.max_tokens - s.num_completion_tokens, self.config.max_model_len - s.num_tokens)
+        if want <= 1:
+            return 1
+        from ..cache import OutOfPages
+        try:
+            for s in seqs:
+                self.runner.cache.reserve(s.seq_id, s.num_tokens + want - 1, first_query=s.num_tokens - 1)
+        except OutOfPages:
+            return 1
+        return want
 
     def generate(self, prompts: Seq[Union[str, List[int]]],
                  sampling_params: Union[SamplingParams, Seq[SamplingParams], None] = None,

@@ -122,13 +122,42 @@ class ModelRunner:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.model.logits(self.model.forward(batch, self.layer_caches), batch.logits_rows)
-            g = (graph, static, logits)
+            g = (graph, static, logits, batch)
             self._graphs[size_b] = g
-        graph, static, logits = g
+        graph, static, logits, _ = g
         build_batch(entries, self.cache, self.page_size, vocab, self.device,
                     table_width=self._graph_table_width, static=static, pad_to=size_b)
         graph.replay()
         return logits[:n]
+
+    @torch.inference_mode()
+    def decode_burst(self, entries: Sequence[StepEntry], steps: int, sampler, temperatures, seeds,
+                     requests) -> List[List[int]]:
+        """`steps` decode steps of the same requests without the host in between: after each
+        captured step the tokens are sampled on the device and a small kernel writes the next
+        step's metadata (tokens, positions, slots) in place.  The entries are the first step's;
+        pages for the positions of all the steps must be reserved.  Returns the sampled tokens,
+        [steps][requests]; they are exactly those of `steps` single steps.  (The reference
+        returns to the host after every step, nanovllm/engine/llm_engine.py:49-55.)"""
+        n = len(entries)
+        if not (self._graph_max_batch and self._graph_takes(entries)):
+            raise ValueError("decode_burst needs captured decode steps and a batch they take")
+        if any(e.start + steps > self._graph_max_len for e in entries):
+            raise ValueError("decode_burst: the steps run past the captured length")
+        self._step_graph(entries)
+        graph, _, logits, batch = self._graphs[self.graph_batch_size(n)]
+        positions = [[e.start + 1 + j for e in entries] for j in range(steps)]
+        temps, keys = sampler.device_inputs(temperatures, seeds, requests, positions)
+        out = torch.empty((steps, n), dtype=torch.int32, device=self.device)
+        kernels = self.model.kernels
+        for j in range(steps):
+            ids = kernels.sample(logits[:n], temps, keys[j])
+            if j + 1 < steps:
+                kernels.advance_decode(batch, ids, out[j], n, self.page_size)
+                graph.replay()
+            else:
+                out[j].copy_(ids)
+        return out.tolist()
 
 
 def load_model(folder: str, dtype: Optional[str] = None, device="cuda:0", kernels=None, quiet: bool = False,

@@ -534,3 +534,27 @@ class HipKernels:
         library.call("sample", None, "nva_sample", _p(logits), c_i64(stride), c_i64(rows), c_i32(vocab),
                      _p(temperatures), _p(keys), _p(out), _p(scratch), self._stream())
         return out
+
+    def advance_decode(self, batch, sampled: torch.Tensor, out_row: torch.Tensor, n_real: int, page_size: int) -> None:
+        """Turns the metadata of a decode step whose tokens were sampled into that of the next
+        decode step of the same requests, in place on the device; out_row receives the tokens."""
+        n_total = batch.num_seqs
+        for t, name in ((batch.input_ids, "input_ids"), (batch.positions, "positions"), (batch.kv_lens, "kv_lens"),
+                        (batch.seq_starts, "seq_starts")):
+            _i32(t, n_total, name)
+        _i32(sampled, n_real, "sampled")
+        _i32(out_row, n_real, "out_row")
+        groups = batch.groups
+        if len(groups) > 4:
+            raise KernelError("advance_decode: at most 4 cache groups")
+        ptr = ctypes.c_void_p * max(len(groups), 1)
+        widths = (ctypes.c_int * max(len(groups), 1))(*[g.block_tables.shape[1] for g in groups])
+        for g in groups:
+            _i32(g.slot_mapping, n_total, "slot_mapping")
+            if g.block_tables.shape[0] != n_total or not g.block_tables.is_contiguous() or g.block_tables.dtype != torch.int32:
+                raise KernelError("advance_decode: block tables must be contiguous int32 [requests, pages]")
+        slots = ptr(*[g.slot_mapping.data_ptr() for g in groups])
+        tables = ptr(*[g.block_tables.data_ptr() for g in groups])
+        library.call("sample", None, "nva_advance_decode", _p(batch.input_ids), _p(batch.positions), _p(batch.kv_lens),
+                     _p(batch.seq_starts), _p(batch.max_kv_dev), _p(sampled), _p(out_row), c_i32(n_real), c_i32(n_total),
+                     c_i32(page_size), c_i32(len(groups)), slots, tables, widths, _p(self.fault_flag), self._stream())

@@ -50,19 +50,28 @@ class Sampler:
         self._temps = None            # (tuple of temperatures, device tensor)
         self._zero_keys = None
 
+    def device_inputs(self, temperatures: Sequence[float], seeds: Sequence[int], requests: Sequence[int],
+                      positions: Sequence[Sequence[int]]):
+        """(temperatures float32 [n], keys int64 [len(positions), n]) on the device, for draws
+        at each of the given rows of positions."""
+        n = len(temperatures)
+        temps = tuple(float(t) for t in temperatures)
+        assert len(seeds) == n and len(requests) == n and all(len(p) == n for p in positions)
+        if self._temps is None or self._temps[0] != temps:
+            self._temps = (temps, torch.tensor(temps, dtype=torch.float32).to(self.device))
+        rows = len(positions)
+        if any(t > 0.0 for t in temps):
+            keys = np.stack([noise_keys(seeds, requests, p) for p in positions])
+            keys_t = torch.from_numpy(keys).to(self.device)
+        else:
+            if self._zero_keys is None or self._zero_keys.numel() < rows * n:
+                self._zero_keys = torch.zeros(max(rows * n, 64), dtype=torch.int64, device=self.device)
+            keys_t = self._zero_keys[:rows * n].view(rows, n)
+        return self._temps[1], keys_t
+
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
                requests: Sequence[int], positions: Sequence[int]) -> List[int]:
         """One token per row of logits.  positions: the position the new token will take."""
-        n = logits.shape[0]
-        temps = tuple(float(t) for t in temperatures)
-        assert len(temps) == n and len(seeds) == n and len(requests) == n and len(positions) == n
-        if self._temps is None or self._temps[0] != temps:
-            self._temps = (temps, torch.tensor(temps, dtype=torch.float32).to(self.device))
-        if any(t > 0.0 for t in temps):
-            keys_t = torch.from_numpy(noise_keys(seeds, requests, positions)).to(self.device)
-        else:
-            if self._zero_keys is None or self._zero_keys.shape[0] < n:
-                self._zero_keys = torch.zeros(max(n, 64), dtype=torch.int64, device=self.device)
-            keys_t = self._zero_keys[:n]
-        ids = self.kernels.sample(logits, self._temps[1], keys_t)
-        return ids.tolist()
+        assert logits.shape[0] == len(temperatures)
+        temps, keys = self.device_inputs(temperatures, seeds, requests, [positions])
+        return self.kernels.sample(logits, temps, keys[0]).tolist()

@@ -112,3 +112,25 @@ def test_throughput_command_with_weights_drawn_on_the_device(tmp_path, capsys):
     assert lines[-2].startswith("Total: ") and "Throughput: " in lines[-2]
     stats = json.loads(lines[-1])
     assert stats["num_seqs"] == 11 and stats["decode_tokens"] > 0 and stats["prefill_tokens"] >= stats["prompt_tokens"]
+
+
+def test_decode_bursts_do_not_change_the_tokens():
+    """Generation with several decode steps in a row on the device (the default) against one step
+    at a time: greedy and at a temperature, requests that end inside a burst by max_tokens and by
+    an eos token, and a pool so small that bursts fall back to single steps."""
+    name, dtype = "c", "bfloat16"
+    prompts = [H.random_tokens(1000, n, 300 + n) for n in (12, 33, 57, 8)]
+    params = [SamplingParams(temperature=t, max_tokens=m) for t, m in ((0.0, 23), (0.7, 9), (1.1, 30), (0.0, 14))]
+    base = _llm(name, dtype, decode_burst=1, max_num_batched_tokens=256).generate(prompts, params, use_tqdm=False)
+    eos = base[2]["token_ids"][11]                                  # request 2 ends here when this token ends requests
+    for kw in (dict(), dict(eos=eos), dict(num_kvcache_blocks=9)):
+        one = base if not kw else _llm(name, dtype, decode_burst=1, max_num_batched_tokens=256, **kw).generate(
+            prompts, params, use_tqdm=False)
+        llm = _llm(name, dtype, decode_burst=6, max_num_batched_tokens=256, **kw)
+        many = llm.generate(prompts, params, use_tqdm=False)
+        assert [o["token_ids"] for o in many] == [o["token_ids"] for o in one], kw
+        if "num_kvcache_blocks" not in kw:                          # (a preempted request gets a token from a prompt step)
+            assert llm.stats["decode_tokens"] == sum(len(o["token_ids"]) for o in many) - len(prompts)
+        else:
+            assert llm.scheduler.num_preemptions > 0
+    assert len(_llm(name, dtype, decode_burst=6, eos=eos).generate(prompts, params, use_tqdm=False)[2]["token_ids"]) <= 12

@@ -58,3 +58,52 @@ def test_graph_replays_equal_eager_steps(name, dtype):
     want = H.plain_logits(folder, reqs["r0"][:pos["r0"]], None if dtype == "float32" else "bfloat16")
     assert H.rel_err(outs[1][0].cpu(), want[-1]) < (2e-5 if dtype == "float32" else 2e-2)
     graphed.kernels.check_faults()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_burst_of_decode_steps_gives_the_tokens_of_single_steps(dtype):
+    """Several captured steps in a row with sampling and the next step's metadata made on the
+    device: the same tokens as step by step through the host, across page edges, with a row of
+    padding, greedy and at a temperature."""
+    from nano_vllm_amd.sampling.sampler import Sampler
+    c = H.CONFIGS["b"]
+    folder = H.model_folder("b", dtype)
+    V = c["cfg"].vocab_size
+    reqs = {i: H.random_tokens(V, n, 60 + i) for i, n in enumerate((21, 30, 13))}
+    temps, seeds = [0.0, 0.8, 1.3], [5, 5, 11]
+    runs = []
+    for burst in (False, True):
+        r = H.make_runner(folder, dtype, c["page"], 64)
+        r.enable_decode_graphs(max_batch=8, max_len=c["cfg"].max_position_embeddings)
+        sampler = Sampler(r.kernels, r.device)
+        toks = {}
+        for rid, t in reqs.items():
+            r.cache.admit(rid)
+            r.cache.reserve(rid, len(t))
+            logits = r.step([StepEntry(rid, t, 0, [len(t) - 1])])
+            toks[rid] = list(t) + sampler.sample(logits, [temps[rid]], [seeds[rid]], [rid], [len(t)])
+        steps = 19                                                  # pages of 8: every request crosses two edges
+        if burst:
+            for lo, n in ((0, 7), (7, 1), (8, 11)):                 # three bursts, one of a single step
+                entries = []
+                for rid in reqs:
+                    r.cache.reserve(rid, len(toks[rid]) + n - 1)
+                    entries.append(StepEntry(rid, [toks[rid][-1]], len(toks[rid]) - 1, [0]))
+                out = r.decode_burst(entries, n, sampler, temps, seeds, list(reqs))
+                for row in out:
+                    for rid, tok in zip(reqs, row):
+                        toks[rid].append(tok)
+        else:
+            for _ in range(steps):
+                entries = []
+                for rid in reqs:
+                    r.cache.reserve(rid, len(toks[rid]))
+                    entries.append(StepEntry(rid, [toks[rid][-1]], len(toks[rid]) - 1, [0]))
+                logits = r.step(entries)
+                out = sampler.sample(logits, temps, seeds, list(reqs), [len(toks[rid]) for rid in reqs])
+                for rid, tok in zip(reqs, out):
+                    toks[rid].append(tok)
+        r.kernels.check_faults()
+        runs.append(toks)
+    assert runs[0] == runs[1]
+    assert all(len(runs[1][rid]) == len(reqs[rid]) + 1 + 19 for rid in reqs)
