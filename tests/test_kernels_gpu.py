@@ -10,6 +10,7 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
+from nano_vllm_amd.kernels.ops import v_cache_shape
 from torch_kernels import TorchKernels, new_caches
 
 pytestmark = pytest.mark.gpu
@@ -370,6 +371,52 @@ def test_paged_attention(hip, ref, dtype, hq, hkv, D, page, lens, q_lens, window
             _close(hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window), twin, dtype, "general")
         finally:
             hip[dtype].mfma_attention = True
+
+
+@pytest.mark.parametrize("page,lens,q_lens,window", [
+    (256, [40000, 12345, 257, 4096], [1, 1, 1, 1], None),           # long decoding: 157 pages in a table
+    (16, [30000, 5000], [1, 1], None),                              # the same over small pages: splits capped by pages
+    (256, [9000, 20000], [1, 700], None),                           # a portion after a long cached prefix
+    (64, [33000], [1500], 4096),                                    # a window far into a long request
+    (256, [16000, 16000, 16000], [1, 1, 300], 1000),
+])
+def test_attention_over_long_contexts_matrix_core_kernels_against_the_general_kernel(hip, page, lens, q_lens, window):
+    """Tens of thousands of keys: the bfloat16 matrix-core kernels (decode with splits, prefill
+    with its block table in LDS) against the general kernel, which the short cases above pin to
+    the plain implementation.  The cache is filled directly; the tables are a random permutation."""
+    hq, hkv, D = 8, 2, 128
+    k = hip[torch.bfloat16]
+    S = len(lens)
+    pages_per = [(n + page - 1) // page for n in lens]
+    total = sum(pages_per) + 5
+    gen = torch.Generator(device=DEV).manual_seed(77)
+    kc = torch.randn((total, hkv, page, D), generator=gen, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    vc = torch.randn(v_cache_shape(total, hkv, D, page), generator=gen, device=DEV, dtype=torch.float32).to(torch.bfloat16)
+    perm = torch.randperm(total).tolist()
+    tables = torch.full((S, max(pages_per)), -1, dtype=torch.int32)
+    token_seq, positions = [], []
+    for s_, n in enumerate(lens):
+        tables[s_, :pages_per[s_]] = torch.tensor([perm.pop() for _ in range(pages_per[s_])], dtype=torch.int32)
+        token_seq += [s_] * q_lens[s_]
+        positions += list(range(n - q_lens[s_], n))
+    assert sorted(q_lens, key=lambda n: n != 1) == list(q_lens)     # single tokens first, as the engine orders a step
+    T = sum(q_lens)
+    q = (torch.randn((T, hq * D), generator=gen, device=DEV, dtype=torch.float32) * 2).to(torch.bfloat16)
+    batch = SimpleNamespace(
+        num_seqs=S, num_tokens=T, token_seq=torch.tensor(token_seq, dtype=torch.int32, device=DEV),
+        positions=torch.tensor(positions, dtype=torch.int32, device=DEV), max_kv_len=max(lens), max_q_len=max(q_lens),
+        kv_lens=torch.tensor(lens, dtype=torch.int32, device=DEV),
+        cu_seqlens_q=torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=DEV),
+        num_decode=next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens)), q_lens=list(q_lens),
+        groups=[SimpleNamespace(block_tables=tables.to(DEV), slot_mapping=None)])
+    got = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, D ** -0.5, window)
+    k.mfma_attention = False
+    try:
+        want = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, D ** -0.5, window)
+    finally:
+        k.mfma_attention = True
+    _close(got, want, torch.bfloat16, "matrix-core kernels against the general kernel")
+    k.check_faults()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
