@@ -117,8 +117,7 @@ class Qwen3Config:
             max_position_embeddings=_require(d, "max_position_embeddings", int, where),
             tie_word_embeddings=bool(d.get("tie_word_embeddings", False)),
             # The reference's getattr default is True (qwen3.py:133); every Qwen3 file
-            # states false and BASELINE configs state "no attention bias", so an absent
-            # key means no bias here.
+            # states false, so an absent key means no bias here.
             attention_bias=bool(d.get("attention_bias", False)),
             hidden_act=act,
             dtype=dtype,

@@ -17,7 +17,7 @@ from nano_vllm_amd.weights import write_random_model
 
 import plain_qwen3 as plain
 
-# Two BASELINE configurations and two more; together they differ in every size and option:
+# Four tiny configurations; together they differ in every size and option:
 # layers, width, heads and groups, head size, inner size, vocabulary, theta, eps, tying,
 # norm weights, page size.
 CONFIGS: Dict[str, dict] = {
