@@ -58,11 +58,11 @@ def main():
     from nano_vllm_amd.sampling.sampler import Sampler
     from nano_vllm_amd.weights import fill_random_
 
-    full_layers = 36
-    cfg = Qwen3Config(vocab_size=151936, hidden_size=4096, num_hidden_layers=args.layers, num_attention_heads=32,
-                      num_key_value_heads=8, head_dim=128, intermediate_size=12288, rms_norm_eps=1e-6,
-                      rope_theta=1000000.0, max_position_embeddings=40960, tie_word_embeddings=False,
-                      dtype=args.dtype)
+    from nano_vllm_amd.models.shapes import shape
+    config_json = shape("qwen3-8b")                      # the benchmark's model: layer sizes of Qwen3-8B
+    full_layers = config_json["num_hidden_layers"]
+    config_json.update(num_hidden_layers=args.layers, torch_dtype=args.dtype)
+    cfg = Qwen3Config.from_dict(config_json)
     device = "cuda:0"
     dtype = torch_dtype(args.dtype)
     itemsize = 2 if args.dtype == "bfloat16" else 4

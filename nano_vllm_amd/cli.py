@@ -92,8 +92,24 @@ def cmd_throughput(args) -> int:
 
 def cmd_random_model(args) -> int:
     from .weights import write_random_model
-    with open(args.config) as f:
-        config = json.load(f)
+    import os
+    if (args.config is None) == (args.shape is None):
+        print("give either --config FILE or --shape NAME", file=sys.stderr)
+        return 2
+    if args.shape is not None:
+        from .models.shapes import shape
+        config = shape(args.shape)
+    else:
+        with open(args.config) as f:
+            config = json.load(f)
+    if args.config_only:                 # for engines started with random_weights: the weights are drawn on the device
+        if args.dtype:
+            config["torch_dtype"] = args.dtype
+        os.makedirs(args.out, exist_ok=True)
+        with open(os.path.join(args.out, "config.json"), "w") as f:
+            json.dump(config, f, indent=2)
+        print(f"wrote {args.out}/config.json")
+        return 0
     write_random_model(args.out, config, args.seed, std=args.std, norm_std=args.norm_std, dtype=args.dtype)
     print(f"wrote {args.out}/config.json and {args.out}/model.safetensors")
     return 0
@@ -124,7 +140,9 @@ def main(argv=None) -> int:
     t.add_argument("--json", action="store_true", help="also print the counts as one JSON line")
     t.set_defaults(fn=cmd_throughput)
     r = sub.add_parser("random-model", help="write a model folder with seeded random weights")
-    r.add_argument("--config", required=True, help="a config.json of the architecture")
+    r.add_argument("--config", default=None, help="a config.json of the architecture")
+    r.add_argument("--shape", default=None, help="a named shape instead: tiny-a, tiny-b, qwen3-8b, qwen3-14b, qwen3-32b")
+    r.add_argument("--config-only", action="store_true", help="write config.json only (for --random-weights)")
     r.add_argument("--seed", type=int, default=0)
     r.add_argument("--out", required=True)
     r.add_argument("--std", type=float, default=0.02)
