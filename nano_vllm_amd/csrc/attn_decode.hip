@@ -63,18 +63,20 @@ __device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf1
     for (int dt = 0; dt < DT; ++dt) vf[dt] = *reinterpret_cast<const bf16x8*>(pv + (int64_t)dt * 16 * vt);
 }
 
-// Keys per split: the longest split that still gives the GPU about 2048 waves when the longest
-// request of the step holds `longest` keys, at least 64 (32 where pages are tiny: a wave keeps its
-// split's block table entries in one register per lane, at most 62 pages).  The launcher and the
-// kernels share this function: a captured launch covers every length up to a bound, and the kernels
-// cut the splits for the step's real longest request, which they read from device memory.
+// Keys per split.  With `tokens` single tokens and kv_heads kv heads, the longest request is cut
+// into as many splits as it takes to give the GPU about 2048 waves (`wanted`), of equal length, a
+// multiple of 32 and at least 64 keys (32 where pages are tiny: a wave keeps its split's block table
+// entries in one register per lane, at most 62 pages).  So a request never has more than `wanted`
+// splits unless the page limit cuts them shorter, whatever its length: a captured launch, which must
+// cover every length up to a bound, is no wider than the launch for the bound itself (workgroups
+// without keys are not free: a grid a few times too wide was measured to double the kernel's time).
+// The launcher and the kernels share this function; the kernels of a captured launch cut the splits
+// for the step's real longest request, which they read from device memory.
 __host__ __device__ inline int nva_decode_split_len(int longest, int tokens, int kv_heads, int page_size) {
-    int len = 64;
-    for (int cand = 8192; cand >= 128; cand >>= 1)
-        if ((int64_t)tokens * kv_heads * ((longest + cand - 1) / cand) >= 2048) {
-            len = cand;
-            break;
-        }
+    const int64_t rows = (int64_t)tokens * kv_heads;
+    const int wanted = (int)((2048 + rows - 1) / rows);
+    int len = ((longest + wanted - 1) / wanted + DEC_CHUNK - 1) / DEC_CHUNK * DEC_CHUNK;
+    if (len < 2 * DEC_CHUNK) len = 2 * DEC_CHUNK;
     const int cap = (62 * page_size) / DEC_CHUNK * DEC_CHUNK;
     if (len > cap) len = cap;
     return len < DEC_CHUNK ? DEC_CHUNK : len;
