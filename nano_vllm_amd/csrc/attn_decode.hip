@@ -4,9 +4,9 @@
 // Semantics as in attn_generic.hip (nanovllm/layers/attention.py:71-74, causal).  The token at
 // position p reads keys first..p, first = max(0, p - window + 1) with a window, else 0.
 //
-// Work split: one wave per (split of the context, kv head, token).  The G = Hq / Hkv query heads
-// of a kv head share its keys: they are the 16 columns of a 16x16x32 MFMA (columns >= G idle).
-// A wave walks its split in chunks of 32 keys:
+// Work split: an item is (split of a token's context, kv head); persistent waves take the items in
+// turn (see decode_plan below).  The G = Hq / Hkv query heads of a kv head share its keys: they are
+// the 16 columns of a 16x16x32 MFMA (columns >= G idle).  A wave walks its split in chunks of 32 keys:
 //   S^T[32 keys x 16 heads] = K[32 x D] Q^T          2 tiles x D/32 MFMAs, K rows straight from global
 //   online softmax over keys (in-lane, then across the 4 lane groups)
 //   O^T[D x 16 heads] += V^T[D x 32 keys] P^T        D/16 MFMAs; P stays in registers
@@ -14,7 +14,7 @@
 // 16-byte load and a chunk's values one contiguous block; the rows of the two S tiles are interleaved (tile a: keys 8g..8g+3, tile b: 8g+4..8g+7 for
 // lane group g) so that a lane's eight probabilities are exactly the eight keys of that load.
 // Each split writes an unnormalised partial result (max, sum, O); a second kernel merges them.
-// With a single split the first kernel writes the result itself.
+// A token with a single split is written by the first kernel itself.
 //
 // Requires head_dim % 32 == 0 (32..256), G <= 16, page_size % 8 == 0; the launcher refuses
 // anything else and the caller falls back to the general kernel.
@@ -63,48 +63,128 @@ __device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf1
     for (int dt = 0; dt < DT; ++dt) vf[dt] = *reinterpret_cast<const bf16x8*>(pv + (int64_t)dt * 16 * vt);
 }
 
-// Keys per split.  With `tokens` single tokens and kv_heads kv heads, the longest request is cut
-// into as many splits as it takes to give the GPU about 2048 waves (`wanted`), of equal length, a
-// multiple of 32 and at least 64 keys (32 where pages are tiny: a wave keeps its split's block table
-// entries in one register per lane, at most 62 pages).  So a request never has more than `wanted`
-// splits unless the page limit cuts them shorter, whatever its length: a captured launch, which must
-// cover every length up to a bound, is no wider than the launch for the bound itself (workgroups
-// without keys are not free: a grid a few times too wide was measured to double the kernel's time).
-// The launcher and the kernels share this function; the kernels of a captured launch cut the splits
-// for the step's real longest request, which they read from device memory.
-__host__ __device__ inline int nva_decode_split_len(int longest, int tokens, int kv_heads, int page_size) {
+// waves the GPU holds at once: the kernel's registers allow two per SIMD, eight per CU, on 256 CUs
+#define DEC_RESIDENT_WAVES 2048
+#define DEC_MAX_TOKENS 1024        // tokens of one launch: their split counts are summed in LDS by every wave
+
+// The plan of a step's decode attention, made on the device from the tokens' positions by one small
+// kernel per step and cache group (so a captured step follows the lengths of the step it is replayed
+// for), and read by the attention kernels of all the group's layers:
+//   keys per split  = mean visible length / wanted, a multiple of 32, at least 64 (32 with tiny
+//                     pages: a wave keeps its split's block table entries in one register per lane,
+//                     at most 62 pages); wanted = ceil(waves / (tokens * kv_heads)) with `waves` the
+//                     waves the GPU holds at once, four times that where the longest request is
+//                     more than 1.25 times the mean (finer items then level the load);
+//   a token's splits are cut at multiples of that length of the absolute position;
+//   the splits of all tokens, counted through, times the kv heads are the launch's items; wave w
+//   of the W persistent waves (as many as the GPU holds at once) takes items w, w + W, ...
+// Sum over tokens of splits <= tokens * (wanted + 2) (or the page limit's count): the size of the
+// partial results, which the launcher checks through nva_attn_decode_plan.
+// plan: [0] keys per split, [1] total splits, [2 .. 2 + tokens] where each token's splits begin,
+// then per split (token << 16) | index of the split within the token's absolute positions.
+__global__ void __launch_bounds__(NVA_WAVE)
+attn_decode_plan_kernel(const int32_t* __restrict__ positions, int tokens, int kv_heads, int page_size, int window,
+                        int max_total_splits, int32_t* __restrict__ plan, int32_t* error_flag) {
+    const int lane = threadIdx.x;
+    // every lane's tokens' positions, loaded at once (-1: no such token)
+    int pos_r[DEC_MAX_TOKENS / NVA_WAVE];
+#pragma unroll
+    for (int i = 0; i < DEC_MAX_TOKENS / NVA_WAVE; ++i) {
+        const int t = i * NVA_WAVE + lane;
+        pos_r[i] = t < tokens ? positions[t] : -1;
+    }
+    int64_t sum = 0;
+    int longest = 0;
+#pragma unroll
+    for (int i = 0; i < DEC_MAX_TOKENS / NVA_WAVE; ++i)
+        if (pos_r[i] >= 0) {
+            const int visible = window > 0 && pos_r[i] + 1 > window ? window : pos_r[i] + 1;
+            sum += visible;
+            longest = max(longest, visible);
+        }
+#pragma unroll
+    for (int off = NVA_WAVE / 2; off > 0; off >>= 1) {
+        sum += __shfl_xor(sum, off, NVA_WAVE);
+        longest = max(longest, __shfl_xor(longest, off, NVA_WAVE));
+    }
+    const int mean = (int)((sum + tokens - 1) / tokens);
     const int64_t rows = (int64_t)tokens * kv_heads;
-    const int wanted = (int)((2048 + rows - 1) / rows);
-    int len = ((longest + wanted - 1) / wanted + DEC_CHUNK - 1) / DEC_CHUNK * DEC_CHUNK;
+    const int64_t target = (int64_t)longest * 4 > (int64_t)mean * 5 ? 4 * DEC_RESIDENT_WAVES : DEC_RESIDENT_WAVES;
+    const int wanted = (int)((target + rows - 1) / rows);
+    int len = ((mean + wanted - 1) / wanted + DEC_CHUNK - 1) / DEC_CHUNK * DEC_CHUNK;
     if (len < 2 * DEC_CHUNK) len = 2 * DEC_CHUNK;
     const int cap = (62 * page_size) / DEC_CHUNK * DEC_CHUNK;
     if (len > cap) len = cap;
-    return len < DEC_CHUNK ? DEC_CHUNK : len;
+    if (len < DEC_CHUNK) len = DEC_CHUNK;
+    int32_t* begin = plan + 2;
+    int32_t* items = plan + 2 + tokens + 1;
+    int carry = 0;
+#pragma unroll
+    for (int i = 0; i < DEC_MAX_TOKENS / NVA_WAVE; ++i) {
+        if (i * NVA_WAVE >= tokens) break;
+        const int t = i * NVA_WAVE + lane;
+        int c = 0, s0 = 0;
+        if (pos_r[i] >= 0) {
+            const int pos = pos_r[i];
+            const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+            s0 = first / len;
+            c = pos / len - s0 + 1;
+        }
+        int incl = c;
+#pragma unroll
+        for (int off = 1; off < NVA_WAVE; off <<= 1) {
+            const int up = __shfl_up(incl, off, NVA_WAVE);
+            if (lane >= off) incl += up;
+        }
+        const int mine = carry + incl - c;
+        if (t < tokens) {
+            begin[t] = min(mine, max_total_splits);
+            for (int k = 0; k < c; ++k)
+                if (mine + k < max_total_splits) items[mine + k] = (t << 16) | (s0 + k);
+        }
+        carry += __shfl(incl, NVA_WAVE - 1, NVA_WAVE);
+    }
+    if (lane == 0) {
+        if (carry > max_total_splits && error_flag) atomicOr(error_flag, 4);   // cannot be, by the launcher's bound
+        plan[0] = len;
+        plan[1] = min(carry, max_total_splits);
+        begin[tokens] = min(carry, max_total_splits);
+    }
 }
 
 template <int D>
 __global__ void __launch_bounds__(NVA_WAVE)
 attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
-                   float* __restrict__ part_o, float* __restrict__ part_ml,
+                   float* __restrict__ part_o, float* __restrict__ part_ml, const int32_t* __restrict__ plan,
                    const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                    const int32_t* __restrict__ block_tables, int table_stride,
-                   const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
-                   int num_q_heads, int num_kv_heads, int page_size, float scale, int window, int split_len,
-                   int num_splits, const int32_t* __restrict__ longest, int32_t* error_flag) {
-    if (longest) split_len = nva_decode_split_len(*longest, (int)gridDim.z, num_kv_heads, page_size);
+                   const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions, int tokens,
+                   int num_q_heads, int num_kv_heads, int page_size, float scale, int window,
+                   int32_t* error_flag) {
     constexpr int KP = D / 32;          // 16-byte pieces of a key row per lane = MFMAs per S tile
     constexpr int DT = D / 16;          // 16-channel tiles of the output
-    const int split = blockIdx.x, kvh = blockIdx.y;
-    const int64_t t = blockIdx.z;
     const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
     const int G = num_q_heads / num_kv_heads;
+    const int split_len = plan[0], total_splits = plan[1];
+    const int32_t* begin = plan + 2;
+    const int32_t* items = plan + 2 + tokens + 1;
+    // row r of S tile a is key 8*(r/4) + r%4 of the chunk, of tile b the same + 4
+    const int row_key = 8 * (col >> 2) + (col & 3);
+
+    for (int item = blockIdx.x; item < total_splits * num_kv_heads; item += gridDim.x) {
+    // neighbouring waves take neighbouring splits of one kv head: the kv heads of a page lie a power of
+    // two apart in the cache, and waves that stream them side by side meet in the same memory channels
+    const int flat = item % total_splits, kvh = item / total_splits;
+    const int packed = items[flat];
+    const int64_t t = packed >> 16;
+    const int split = packed & 0xffff;
+    const int splits_of_t = begin[t + 1] - begin[t];
     const int pos = positions[t];
     const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
     const int kv_len = pos + 1;
     // the splits are cut at multiples of split_len of the absolute position
     const int lo = max(split * split_len, first & ~(DEC_CHUNK - 1));
     const int hi = min((split + 1) * split_len, kv_len);
-    if (lo >= hi) return;
     const int32_t* table = block_tables + (int64_t)token_seq[t] * table_stride;
 
     // Q: column `col` is query head kvh*G + col; lane group g holds channels [g*D/4, (g+1)*D/4)
@@ -126,10 +206,6 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 #pragma unroll
     for (int i = 0; i < DT; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
-
-    // row r of S tile a is key 8*(r/4) + r%4 of the chunk, of tile b the same + 4
-    const int row_key = 8 * (col >> 2) + (col & 3);
-
     // The loads of chunk i + 1 are issued before the products of chunk i, so that a wave always has
     // a chunk (16 KiB at head_dim 128) in flight.
     // Lane i of the wave keeps block table entry window_page0 + i: a split spans at most 64 pages
@@ -207,49 +283,49 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     }
 
     // acc[dt][i] = O[head col][channel 16*dt + 4*g + i]
-    if (col >= G) return;
-    const int head = kvh * G + col;
-    if (num_splits == 1) {
-        const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
-        __bf16* orow = out + t * out_stride + (int64_t)head * D;
+    if (col < G) {
+        const int head = kvh * G + col;
+        if (splits_of_t == 1) {
+            const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+            __bf16* orow = out + t * out_stride + (int64_t)head * D;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) orow[16 * dt + 4 * g + i] = (__bf16)(acc[dt][i] * inv);
-    } else {
-        const int64_t slot = ((int64_t)t * num_q_heads + head) * num_splits + split;
-        float* po = part_o + slot * D;
+                for (int i = 0; i < 4; ++i) orow[16 * dt + 4 * g + i] = (__bf16)(acc[dt][i] * inv);
+        } else {
+            const int64_t slot = (int64_t)flat * num_q_heads + head;
+            float* po = part_o + slot * D;
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-            *reinterpret_cast<f32x4*>(po + 16 * dt + 4 * g) = acc[dt];
-        if (g == 0) {
-            part_ml[slot * 2] = m_run;
-            part_ml[slot * 2 + 1] = l_run;
+            for (int dt = 0; dt < DT; ++dt)
+                *reinterpret_cast<f32x4*>(po + 16 * dt + 4 * g) = acc[dt];
+            if (g == 0) {
+                part_ml[slot * 2] = m_run;
+                part_ml[slot * 2 + 1] = l_run;
+            }
         }
+    }
     }
 }
 
-// Merges the splits of one (token, head): o = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m).
-// One workgroup of four waves per (token, head).  Every wave finds the maximum m over the visible
-// splits, then takes every fourth group of four splits (their loads overlap) and the four partial
-// sums meet in LDS; the order of the sum depends on the number of splits only.
+// Merges the splits of one (token, head): o = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m); a
+// token with one split was written by the attention kernel itself.  One workgroup of four waves per
+// (token, head).  Every wave finds the maximum m over the splits, then takes every fourth group of
+// four splits (their loads overlap) and the four partial sums meet in LDS; the order of the sum
+// depends on the number of splits only.
 #define MERGE_WAVES 4
 __global__ void __launch_bounds__(MERGE_WAVES * NVA_WAVE)
 attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                         __bf16* __restrict__ out, int64_t out_stride, const int32_t* __restrict__ positions,
-                         int num_q_heads, int num_kv_heads, int page_size, int head_dim, int window, int split_len,
-                         int num_splits, const int32_t* __restrict__ longest) {
-    if (longest) split_len = nva_decode_split_len(*longest, (int)gridDim.x, num_kv_heads, page_size);
+                         const int32_t* __restrict__ plan, __bf16* __restrict__ out, int64_t out_stride,
+                         int num_q_heads, int head_dim) {
     __shared__ float acc_s[MERGE_WAVES][4 * NVA_WAVE];
     __shared__ float l_s[MERGE_WAVES];
     const int64_t t = blockIdx.x;
     const int head = blockIdx.y, lane = threadIdx.x % NVA_WAVE, wave = threadIdx.x / NVA_WAVE;
-    const int pos = positions[t];
-    const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
-    const int s_lo = first / split_len, s_hi = pos / split_len;          // splits that hold visible keys
-    const int64_t slot0 = ((int64_t)t * num_q_heads + head) * num_splits;
+    const int s_lo = plan[2 + t], s_hi = plan[2 + t + 1] - 1;             // the token's splits, counted through
+    if (s_hi <= s_lo) return;
+    auto slot_of = [&](int s) { return (int64_t)s * num_q_heads + head; };
     float m = -INFINITY;
-    for (int s = s_lo + lane; s <= s_hi; s += NVA_WAVE) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
+    for (int s = s_lo + lane; s <= s_hi; s += NVA_WAVE) m = fmaxf(m, part_ml[slot_of(s) * 2]);
     m = wave_max(m);
     float l = 0.f;
     float acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -258,10 +334,10 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int s = min(s0 + j, s_hi);                              // a split past the end: read again, weight 0
-            const float ms = part_ml[(slot0 + s) * 2];
+            const float ms = part_ml[slot_of(s) * 2];
             wj[j] = (s0 + j > s_hi || ms == -INFINITY) ? 0.f : __expf(ms - m);
-            l += part_ml[(slot0 + s) * 2 + 1] * wj[j];
-            const float* po = part_o + (slot0 + s) * head_dim;
+            l += part_ml[slot_of(s) * 2 + 1] * wj[j];
+            const float* po = part_o + slot_of(s) * head_dim;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int d = lane + i * NVA_WAVE;
@@ -293,34 +369,52 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
     }
 }
 
-// What a launch needs for `tokens` single tokens whose longest request holds at most `longest`
-// keys: the keys per split and the number of splits (the grid's width and the stride of the
-// partial results).  lengths_vary: the launch is captured and replayed for every length up to
-// `longest`; the number of splits then covers them all.
-NVA_EXPORT int nva_attn_decode_plan_bf16(int longest, int64_t tokens, int num_kv_heads, int page_size, int lengths_vary,
-                                    int* split_len, int* num_splits) {
-    if (longest <= 0 || tokens <= 0 || tokens > 65535 || num_kv_heads <= 0 || page_size <= 0 || !split_len || !num_splits)
-        return nva_fail("attn_decode_plan: bad arguments");
-    *split_len = nva_decode_split_len(longest, (int)tokens, num_kv_heads, page_size);
-    *num_splits = (longest + *split_len - 1) / *split_len;
-    if (lengths_vary)
-        for (int len = DEC_CHUNK; len < longest; len += DEC_CHUNK) {
-            const int s = nva_decode_split_len(len, (int)tokens, num_kv_heads, page_size);
-            if ((len + s - 1) / s > *num_splits) *num_splits = (len + s - 1) / s;
-        }
+// What the decode attention of `tokens` single tokens needs when no request holds more than `longest`
+// keys: the bound of the splits of all tokens together, the number of persistent waves, and the size
+// of the plan (int32).  Partial results: max_total_splits * num_q_heads * (head_dim + 2) floats.
+NVA_EXPORT int nva_attn_decode_plan_size_bf16(int longest, int64_t tokens, int num_kv_heads, int page_size,
+                                              int* max_total_splits, int* waves, int64_t* plan_ints) {
+    if (longest <= 0 || tokens <= 0 || tokens > DEC_MAX_TOKENS || num_kv_heads <= 0 || page_size <= 0 ||
+        !max_total_splits || !waves || !plan_ints)
+        return nva_fail("attn_decode_plan_size: bad arguments (at most %d tokens a launch)", DEC_MAX_TOKENS);
+    const int64_t rows = tokens * num_kv_heads;
+    const int64_t wanted = (4 * DEC_RESIDENT_WAVES + rows - 1) / rows;
+    // sum of the tokens' counts <= total / len + 2 * tokens; len >= mean / wanted unless the page limit cuts it
+    const int cap = (62 * page_size) / DEC_CHUNK * DEC_CHUNK > DEC_CHUNK ? (62 * page_size) / DEC_CHUNK * DEC_CHUNK : DEC_CHUNK;
+    int64_t per_token = wanted;
+    if ((longest + cap - 1) / cap > per_token) per_token = (longest + cap - 1) / cap;
+    if (per_token > (longest + DEC_CHUNK - 1) / DEC_CHUNK) per_token = (longest + DEC_CHUNK - 1) / DEC_CHUNK;
+    const int64_t bound = tokens * (per_token + 2);
+    if (bound * num_kv_heads > 0x7fffffff || (longest + DEC_CHUNK - 1) / DEC_CHUNK > 0xffff)
+        return nva_fail("attn_decode_plan_size: too many splits");
+    *max_total_splits = (int)bound;
+    const int64_t items = bound * num_kv_heads;
+    *waves = (int)(items < DEC_RESIDENT_WAVES ? items : DEC_RESIDENT_WAVES);
+    *plan_ints = 2 + tokens + 1 + bound;
     return 0;
 }
 
+// Makes the plan of a step (once per step and cache group; every layer's attention reads it).
+NVA_EXPORT int nva_attn_decode_plan_bf16(const int32_t* positions, int64_t tokens, int num_kv_heads, int page_size,
+                                         int window, int max_total_splits, int32_t* plan, int32_t* error_flag,
+                                         hipStream_t stream) {
+    if (!positions || !plan || tokens <= 0 || tokens > DEC_MAX_TOKENS || num_kv_heads <= 0 || page_size <= 0 ||
+        window < 0 || max_total_splits <= 0)
+        return nva_fail("attn_decode_plan: bad arguments");
+    hipLaunchKernelGGL(attn_decode_plan_kernel, dim3(1), dim3(NVA_WAVE), 0, stream, positions, (int)tokens, num_kv_heads,
+                       page_size, window, max_total_splits, plan, error_flag);
+    return nva_check_launch("attn_decode_plan");
+}
+
 // Returns 1 (and leaves a message) for shapes this kernel does not take; the caller then uses the
-// general kernel.  split_len and num_splits come from nva_attn_decode_plan.  longest: null, or a
-// device int32 with the keys of the step's longest request, from which the kernels then cut the
-// splits themselves (a captured launch, planned with lengths_vary).
+// general kernel.  plan: made by nva_attn_decode_plan for these tokens, kv heads, page size and
+// window; max_total_splits and waves from nva_attn_decode_plan_size.
 NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride, float* scratch,
-                                    const void* k_cache, const void* v_cache, const int32_t* block_tables,
-                                    int table_stride, const int32_t* token_seq, const int32_t* positions,
-                                    int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, int page_size,
-                                    float scale, int window, int split_len, int num_splits, const int32_t* longest,
-                                    int32_t* error_flag, hipStream_t stream) {
+                                    const int32_t* plan, const void* k_cache, const void* v_cache,
+                                    const int32_t* block_tables, int table_stride, const int32_t* token_seq,
+                                    const int32_t* positions, int64_t tokens, int num_q_heads, int num_kv_heads,
+                                    int head_dim, int page_size, float scale, int window, int max_total_splits,
+                                    int waves, int32_t* error_flag, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_decode: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
@@ -330,21 +424,19 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
                  "page_size %% 8 == 0 (got head_dim %d, group %d, page %d)", head_dim, G, page_size);
         return 1;
     }
-    if (tokens < 0 || tokens > 65535 || num_kv_heads > 65535)
-        return nva_fail("attn_decode: %lld tokens or %d kv heads exceed the grid", (long long)tokens, num_kv_heads);
-    if (split_len <= 0 || split_len % DEC_CHUNK || num_splits <= 0 || window < 0 || table_stride <= 0)
-        return nva_fail("attn_decode: bad split_len %d / num_splits %d / window %d", split_len, num_splits, window);
-    if (split_len / page_size + 2 > NVA_WAVE)
-        return nva_fail("attn_decode: a split of %d keys spans more than %d pages of %d", split_len, NVA_WAVE - 2, page_size);
-    if (num_splits > 1 && !scratch) return nva_fail("attn_decode: several splits need scratch memory");
+    if (tokens < 0 || tokens > DEC_MAX_TOKENS || num_q_heads > 65535)
+        return nva_fail("attn_decode: %lld tokens (at most %d a launch) or %d heads exceed the grid", (long long)tokens,
+                        DEC_MAX_TOKENS, num_q_heads);
+    if (max_total_splits <= 0 || waves <= 0 || window < 0 || table_stride <= 0 || !scratch || !plan)
+        return nva_fail("attn_decode: bad plan (%d splits, %d waves), window %d or no scratch", max_total_splits, waves,
+                        window);
     float* part_o = scratch;
-    float* part_ml = scratch ? scratch + tokens * num_q_heads * (int64_t)num_splits * head_dim : nullptr;
-    dim3 grid((unsigned)num_splits, (unsigned)num_kv_heads, (unsigned)tokens);
+    float* part_ml = scratch + (int64_t)max_total_splits * num_q_heads * head_dim;
 #define LAUNCH(DD)                                                                                              \
-    hipLaunchKernelGGL(attn_decode_kernel<DD>, grid, dim3(NVA_WAVE), 0, stream, (const __bf16*)q, q_stride,       \
-                       (__bf16*)out, out_stride, part_o, part_ml, (const __bf16*)k_cache, (const __bf16*)v_cache, \
-                       block_tables, table_stride, token_seq, positions, num_q_heads, num_kv_heads, page_size,    \
-                       scale, window, split_len, num_splits, longest, error_flag)
+    hipLaunchKernelGGL(attn_decode_kernel<DD>, dim3((unsigned)waves), dim3(NVA_WAVE), 0, stream, (const __bf16*)q, \
+                       q_stride, (__bf16*)out, out_stride, part_o, part_ml, plan, (const __bf16*)k_cache,         \
+                       (const __bf16*)v_cache, block_tables, table_stride, token_seq, positions, (int)tokens,     \
+                       num_q_heads, num_kv_heads, page_size, scale, window, error_flag)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;
@@ -359,14 +451,10 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
 #undef LAUNCH
     int rc = nva_check_launch("attn_decode");
     if (rc) return rc;
-    if (num_splits > 1) {
-        dim3 mgrid((unsigned)tokens, (unsigned)num_q_heads);
-        hipLaunchKernelGGL(attn_decode_merge_kernel, mgrid, dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, (__bf16*)out,
-                           out_stride, positions, num_q_heads, num_kv_heads, page_size, head_dim, window, split_len,
-                           num_splits, longest);
-        rc = nva_check_launch("attn_decode_merge");
-    }
-    return rc;
+    dim3 mgrid((unsigned)tokens, (unsigned)num_q_heads);
+    hipLaunchKernelGGL(attn_decode_merge_kernel, mgrid, dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, plan,
+                       (__bf16*)out, out_stride, num_q_heads, head_dim);
+    return nva_check_launch("attn_decode_merge");
 }
 
 NVA_DEFINE_LAST_ERROR(nva_attn_decode)

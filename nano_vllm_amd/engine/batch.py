@@ -53,7 +53,8 @@ class StepBatch:
     q_lens: List[int] = field(default_factory=list)
     starts: List[int] = field(default_factory=list)
     requests: List[Hashable] = field(default_factory=list)
-    lengths_vary: bool = False       # a captured launch: max_kv_len is a bound, max_kv_dev the step's value
+    lengths_vary: bool = False       # a captured launch: max_kv_len is a bound of the steps it is replayed for
+    step_cache: dict = field(default_factory=dict)   # emptied by the model at the start of every pass
 
 
 def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size: int, device,

@@ -491,28 +491,33 @@ class HipKernels:
 
     def _attention_decode(self, q, qs, out, os_, k_cache, v_cache, tables, batch, n, num_heads, num_kv_heads,
                           head_dim, page_size, scale, window):
-        # keys per split and number of splits: the kernels' own rule (one place, in the library).  A
-        # batch that a captured graph replays covers every length up to its bound, and the kernels read
-        # the step's longest request from the batch's device copy.
-        vary = bool(getattr(batch, "lengths_vary", False))
-        longest = getattr(batch, "max_kv_dev", None) if vary else None
-        if vary and (longest is None or n > 65535):
-            raise KernelError("attention: a batch whose lengths vary needs max_kv_dev and at most 65535 tokens")
-        split_len, num_splits = ctypes.c_int(0), ctypes.c_int(0)
-        library.call("attn_decode", "bf16", "nva_attn_decode_plan", c_i32(batch.max_kv_len), c_i64(min(n, 65535)),
-                     c_i32(num_kv_heads), c_i32(page_size), c_i32(1 if vary else 0), ctypes.byref(split_len),
-                     ctypes.byref(num_splits))
-        split_len, num_splits = split_len.value, num_splits.value
-        scratch = None
-        if num_splits > 1:
-            scratch = torch.empty(n * num_heads * num_splits * (head_dim + 2), dtype=torch.float32, device=q.device)
-        for t0 in range(0, n, 65535):                               # grid.z holds at most 65535 tokens
-            t1 = min(n, t0 + 65535)
+        # The splits are planned on the device from the tokens' positions, once per step and (kv
+        # heads, window): the first layer that asks makes the plan, the others find it on the batch.
+        # The library says how large the partial results may get for this many tokens of at most
+        # max_kv_len keys, and how many persistent waves to launch.  At most 1024 tokens a launch.
+        plans = getattr(batch, "step_cache", None)         # emptied by the model at the start of every pass
+        if plans is None:
+            plans = batch.step_cache = {}
+        for t0 in range(0, n, 1024):
+            t1 = min(n, t0 + 1024)
+            key = ("decode_plan", t0, num_kv_heads, page_size, window or 0)
+            if key not in plans:
+                bound, waves, ints = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int64(0)
+                library.call("attn_decode", "bf16", "nva_attn_decode_plan_size", c_i32(batch.max_kv_len), c_i64(t1 - t0),
+                             c_i32(num_kv_heads), c_i32(page_size), ctypes.byref(bound), ctypes.byref(waves),
+                             ctypes.byref(ints))
+                plan = torch.empty(ints.value, dtype=torch.int32, device=q.device)
+                library.call("attn_decode", "bf16", "nva_attn_decode_plan", _p(batch.positions[t0:t1]), c_i64(t1 - t0),
+                             c_i32(num_kv_heads), c_i32(page_size), c_i32(window or 0), c_i32(bound.value), _p(plan),
+                             _p(self.fault_flag), self._stream())
+                plans[key] = (plan, bound.value, waves.value)
+            plan, bound, waves = plans[key]
+            scratch = torch.empty(bound * num_heads * (head_dim + 2), dtype=torch.float32, device=q.device)
             library.call("attn_decode", "bf16", "nva_attn_decode", _p(q[t0:t1]), c_i64(qs), _p(out[t0:t1]), c_i64(os_),
-                         _p(scratch), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
+                         _p(scratch), _p(plan), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          _p(batch.token_seq[t0:t1]), _p(batch.positions[t0:t1]), c_i64(t1 - t0), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
-                         c_i32(split_len), c_i32(num_splits), _p(longest), _p(self.fault_flag), self._stream())
+                         c_i32(bound), c_i32(waves), _p(self.fault_flag), self._stream())
 
     # ------------------------------------------------------------------ sampling
     def sample(self, logits: torch.Tensor, temperatures: torch.Tensor, keys: torch.Tensor) -> torch.Tensor:

@@ -128,6 +128,7 @@ class Model:
     # ------------------------------------------------------------------ forward
     def forward(self, batch, caches: List[LayerCache]) -> torch.Tensor:
         """Hidden states [T, hidden] of the batch's tokens after the final norm."""
+        batch.step_cache = {}        # what kernels share between the layers of one pass (a plan made by the first)
         h = self.embedding.forward(batch.input_ids)
         residual = None
         for i, run in enumerate(self.order):
