@@ -4,17 +4,17 @@
 // Semantics as in attn_generic.hip (nanovllm/layers/attention.py:71-74, causal).  The token at
 // position p reads keys first..p, first = max(0, p - window + 1) with a window, else 0.
 //
-// Work split: an item is (split of a token's context, kv head); persistent waves take the items in
-// turn (see decode_plan below).  The G = Hq / Hkv query heads of a kv head share its keys: they are
-// the 16 columns of a 16x16x32 MFMA (columns >= G idle).  A wave walks its split in chunks of 32 keys:
+// Work split: the keys that the step's tokens see are cut into equal quotas, one per wave and kv
+// head (see the plan below).  The G = Hq / Hkv query heads of a kv head share its keys: they are
+// the 16 columns of a 16x16x32 MFMA (columns >= G idle).  A wave walks its keys in chunks of 32:
 //   S^T[32 keys x 16 heads] = K[32 x D] Q^T          2 tiles x D/32 MFMAs, K rows straight from global
 //   online softmax over keys (in-lane, then across the 4 lane groups)
 //   O^T[D x 16 heads] += V^T[D x 32 keys] P^T        D/16 MFMAs; P stays in registers
 // The transposed V cache (tiles [D, 32 keys], common.h) makes 8 consecutive keys of one channel one
 // 16-byte load and a chunk's values one contiguous block; the rows of the two S tiles are interleaved (tile a: keys 8g..8g+3, tile b: 8g+4..8g+7 for
 // lane group g) so that a lane's eight probabilities are exactly the eight keys of that load.
-// Each split writes an unnormalised partial result (max, sum, O); a second kernel merges them.
-// A token with a single split is written by the first kernel itself.
+// A token whose keys lie in several quotas gets an unnormalised partial result (max, sum, O) from
+// each; a second kernel merges them.  A token inside one quota is written by the first kernel itself.
 //
 // Requires head_dim % 32 == 0 (32..256), G <= 16, page_size % 8 == 0; the launcher refuses
 // anything else and the caller falls back to the general kernel.
@@ -65,161 +65,201 @@ __device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf1
 
 // waves the GPU holds at once: the kernel's registers allow two per SIMD, eight per CU, on 256 CUs
 #define DEC_RESIDENT_WAVES 2048
-#define DEC_MAX_TOKENS 1024        // tokens of one launch: their split counts are summed in LDS by every wave
+#define DEC_MAX_TOKENS 1024        // tokens of one launch: one wave plans them, 16 to a lane
 
 // The plan of a step's decode attention, made on the device from the tokens' positions by one small
 // kernel per step and cache group (so a captured step follows the lengths of the step it is replayed
-// for), and read by the attention kernels of all the group's layers:
-//   keys per split  = mean visible length / wanted, a multiple of 32, at least 64 (32 with tiny
-//                     pages: a wave keeps its split's block table entries in one register per lane,
-//                     at most 62 pages); wanted = ceil(waves / (tokens * kv_heads)) with `waves` the
-//                     waves the GPU holds at once, four times that where the longest request is
-//                     more than 1.25 times the mean (finer items then level the load);
-//   a token's splits are cut at multiples of that length of the absolute position;
-//   the splits of all tokens, counted through, times the kv heads are the launch's items; wave w
-//   of the W persistent waves (as many as the GPU holds at once) takes items w, w + W, ...
-// Sum over tokens of splits <= tokens * (wanted + 2) (or the page limit's count): the size of the
-// partial results, which the launcher checks through nva_attn_decode_plan.
-// plan: [0] keys per split, [1] total splits, [2 .. 2 + tokens] where each token's splits begin,
-// then per split (token << 16) | index of the split within the token's absolute positions.
+// for), and read by the attention kernels of all the group's layers.
+//
+// Every wave gets the same amount of work, whatever the lengths of the requests: the chunks (32
+// keys) that the tokens see are counted through, token after token, and cut into quotas of equal
+// size, one quota for each of the W waves that work on a kv head (W = waves of the launch / kv
+// heads, as many as the GPU holds at once); at least two chunks a quota, and at most what 62 pages
+// hold (a wave keeps the block table entries of what it reads in one register per lane), in which
+// case a wave takes several quotas in turn.  A quota is one or more segments: (token, keys lo..hi).
+// A token cut by a quota's edge has several segments, which a second kernel merges; a token with
+// one segment is written by the attention kernel itself.  Segments <= tokens + quotas.
+//
+// plan (int32): [0] number of quotas, [1] number of segments, [2 .. 2 + tokens] where each token's
+// segments begin; from decode_plan_quotas_at on, the first segment of every quota (and the number
+// of segments after the last); from decode_plan_segments_at on, eight ints per segment: token,
+// its request's block table row, its position, 1 if it is the token's only segment; lo, hi, -, -.
+__host__ __device__ inline int64_t decode_plan_quotas_at(int64_t tokens) { return (2 + tokens + 1 + 3) / 4 * 4; }
+__host__ __device__ inline int64_t decode_plan_segments_at(int64_t tokens, int64_t max_segments) {
+    return (decode_plan_quotas_at(tokens) + (max_segments - tokens) + 2 + 3) / 4 * 4;     // quotas <= segments - tokens
+}
+__host__ __device__ inline int decode_quota_cap(int page_size) {
+    const int cap = (62 * page_size) / DEC_CHUNK;
+    return cap > 1 ? cap : 1;
+}
+
 __global__ void __launch_bounds__(NVA_WAVE)
-attn_decode_plan_kernel(const int32_t* __restrict__ positions, int tokens, int kv_heads, int page_size, int window,
-                        int max_total_splits, int32_t* __restrict__ plan, int32_t* error_flag) {
+attn_decode_plan_kernel(const int32_t* __restrict__ positions, const int32_t* __restrict__ token_seq, int tokens,
+                        int page_size, int window, int max_segments, int waves_per_head, int32_t* __restrict__ plan,
+                        int32_t* error_flag) {
     const int lane = threadIdx.x;
-    // every lane's tokens' positions, loaded at once (-1: no such token)
+    // every lane's tokens: position (-1: no such token) and the chunks it sees
     int pos_r[DEC_MAX_TOKENS / NVA_WAVE];
+    int total = 0;
 #pragma unroll
     for (int i = 0; i < DEC_MAX_TOKENS / NVA_WAVE; ++i) {
         const int t = i * NVA_WAVE + lane;
         pos_r[i] = t < tokens ? positions[t] : -1;
     }
-    int64_t sum = 0;
-    int longest = 0;
 #pragma unroll
     for (int i = 0; i < DEC_MAX_TOKENS / NVA_WAVE; ++i)
         if (pos_r[i] >= 0) {
-            const int visible = window > 0 && pos_r[i] + 1 > window ? window : pos_r[i] + 1;
-            sum += visible;
-            longest = max(longest, visible);
+            const int first = window > 0 && pos_r[i] - window + 1 > 0 ? pos_r[i] - window + 1 : 0;
+            total += pos_r[i] / DEC_CHUNK - first / DEC_CHUNK + 1;
         }
 #pragma unroll
-    for (int off = NVA_WAVE / 2; off > 0; off >>= 1) {
-        sum += __shfl_xor(sum, off, NVA_WAVE);
-        longest = max(longest, __shfl_xor(longest, off, NVA_WAVE));
+    for (int off = NVA_WAVE / 2; off > 0; off >>= 1) total += __shfl_xor(total, off, NVA_WAVE);
+    int quota = (total + waves_per_head - 1) / waves_per_head;
+    if (quota < 2) quota = 2;
+    if (quota > decode_quota_cap(page_size)) quota = decode_quota_cap(page_size);
+    int num_quotas = (total + quota - 1) / quota;
+    const int max_quotas = max_segments - tokens;
+    if (num_quotas > max_quotas) {                       // cannot be, by the launcher's bound
+        if (error_flag && lane == 0) atomicOr(error_flag, 4);
+        num_quotas = 0;
     }
-    const int mean = (int)((sum + tokens - 1) / tokens);
-    const int64_t rows = (int64_t)tokens * kv_heads;
-    const int64_t target = (int64_t)longest * 4 > (int64_t)mean * 5 ? 4 * DEC_RESIDENT_WAVES : DEC_RESIDENT_WAVES;
-    const int wanted = (int)((target + rows - 1) / rows);
-    int len = ((mean + wanted - 1) / wanted + DEC_CHUNK - 1) / DEC_CHUNK * DEC_CHUNK;
-    if (len < 2 * DEC_CHUNK) len = 2 * DEC_CHUNK;
-    const int cap = (62 * page_size) / DEC_CHUNK * DEC_CHUNK;
-    if (len > cap) len = cap;
-    if (len < DEC_CHUNK) len = DEC_CHUNK;
     int32_t* begin = plan + 2;
-    int32_t* items = plan + 2 + tokens + 1;
-    int carry = 0;
+    int32_t* quota_first = plan + decode_plan_quotas_at(tokens);
+    int4* segments = reinterpret_cast<int4*>(plan + decode_plan_segments_at(tokens, max_segments));
+    int chunks_before = 0, segments_before = 0;
 #pragma unroll
     for (int i = 0; i < DEC_MAX_TOKENS / NVA_WAVE; ++i) {
         if (i * NVA_WAVE >= tokens) break;
         const int t = i * NVA_WAVE + lane;
-        int c = 0, s0 = 0;
-        if (pos_r[i] >= 0) {
-            const int pos = pos_r[i];
-            const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
-            s0 = first / len;
-            c = pos / len - s0 + 1;
-        }
+        const int pos = pos_r[i];
+        const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+        const int c = pos >= 0 && num_quotas > 0 ? pos / DEC_CHUNK - first / DEC_CHUNK + 1 : 0;
         int incl = c;
 #pragma unroll
         for (int off = 1; off < NVA_WAVE; off <<= 1) {
             const int up = __shfl_up(incl, off, NVA_WAVE);
             if (lane >= off) incl += up;
         }
-        const int mine = carry + incl - c;
-        if (t < tokens) {
-            begin[t] = min(mine, max_total_splits);
-            for (int k = 0; k < c; ++k)
-                if (mine + k < max_total_splits) items[mine + k] = (t << 16) | (s0 + k);
+        const int cum = chunks_before + incl - c;                   // the token's first chunk, counted through
+        chunks_before += __shfl(incl, NVA_WAVE - 1, NVA_WAVE);
+        const int n = c > 0 ? (cum + c - 1) / quota - cum / quota + 1 : 0;
+        incl = n;
+#pragma unroll
+        for (int off = 1; off < NVA_WAVE; off <<= 1) {
+            const int up = __shfl_up(incl, off, NVA_WAVE);
+            if (lane >= off) incl += up;
         }
-        carry += __shfl(incl, NVA_WAVE - 1, NVA_WAVE);
+        const int mine = segments_before + incl - n;
+        segments_before += __shfl(incl, NVA_WAVE - 1, NVA_WAVE);
+        if (t < tokens) {
+            begin[t] = mine;
+            const int seq = token_seq[t];
+            for (int k = 0; k < n; ++k) {
+                const int qi = cum / quota + k;
+                const int c_lo = max(cum, qi * quota), c_hi = min(cum + c, (qi + 1) * quota);
+                const int lo = (first / DEC_CHUNK + c_lo - cum) * DEC_CHUNK;
+                const int hi = min((first / DEC_CHUNK + c_hi - cum) * DEC_CHUNK, pos + 1);
+                if (mine + k < max_segments) {
+                    segments[2 * (mine + k)] = make_int4(t, seq, pos, n == 1);
+                    segments[2 * (mine + k) + 1] = make_int4(lo, hi, 0, 0);
+                    if (c_lo == qi * quota) quota_first[qi] = mine + k;
+                }
+            }
+        }
     }
     if (lane == 0) {
-        if (carry > max_total_splits && error_flag) atomicOr(error_flag, 4);   // cannot be, by the launcher's bound
-        plan[0] = len;
-        plan[1] = min(carry, max_total_splits);
-        begin[tokens] = min(carry, max_total_splits);
+        plan[0] = num_quotas;
+        plan[1] = segments_before;
+        begin[tokens] = segments_before;
+        quota_first[num_quotas] = segments_before;
     }
 }
 
 template <int D>
-__global__ void __launch_bounds__(NVA_WAVE)
+__global__ void __launch_bounds__(NVA_WAVE) __attribute__((amdgpu_waves_per_eu(D <= 128 ? 2 : 1, 2)))
 attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
                    float* __restrict__ part_o, float* __restrict__ part_ml, const int32_t* __restrict__ plan,
                    const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
-                   const int32_t* __restrict__ block_tables, int table_stride,
-                   const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions, int tokens,
+                   const int32_t* __restrict__ block_tables, int table_stride, int tokens, int max_segments,
                    int num_q_heads, int num_kv_heads, int page_size, float scale, int window,
                    int32_t* error_flag) {
     constexpr int KP = D / 32;          // 16-byte pieces of a key row per lane = MFMAs per S tile
     constexpr int DT = D / 16;          // 16-channel tiles of the output
     const int lane = threadIdx.x, col = lane & 15, g = lane >> 4;
     const int G = num_q_heads / num_kv_heads;
-    const int split_len = plan[0], total_splits = plan[1];
-    const int32_t* begin = plan + 2;
-    const int32_t* items = plan + 2 + tokens + 1;
+    // Neighbouring waves take neighbouring quotas of one kv head: the kv heads of a page lie a power
+    // of two apart in the cache, and waves that stream them side by side meet in the same memory
+    // channels.
+    const int waves_per_head = gridDim.x / num_kv_heads;
+    const int kvh = blockIdx.x / waves_per_head;
+    int quota = blockIdx.x % waves_per_head;
+    const int32_t* quota_first = plan + decode_plan_quotas_at(tokens);
+    const int4* segments = reinterpret_cast<const int4*>(plan + decode_plan_segments_at(tokens, max_segments));
+    int seg = quota_first[quota], seg_end = quota_first[quota + 1];      // read before it is known that the quota exists
+    const int num_quotas = plan[0];
+    if (quota >= num_quotas) return;
     // row r of S tile a is key 8*(r/4) + r%4 of the chunk, of tile b the same + 4
     const int row_key = 8 * (col >> 2) + (col & 3);
 
-    for (int item = blockIdx.x; item < total_splits * num_kv_heads; item += gridDim.x) {
-    // neighbouring waves take neighbouring splits of one kv head: the kv heads of a page lie a power of
-    // two apart in the cache, and waves that stream them side by side meet in the same memory channels
-    const int flat = item % total_splits, kvh = item / total_splits;
-    const int packed = items[flat];
-    const int64_t t = packed >> 16;
-    const int split = packed & 0xffff;
-    const int splits_of_t = begin[t + 1] - begin[t];
-    const int pos = positions[t];
-    const int first = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
-    const int kv_len = pos + 1;
-    // the splits are cut at multiples of split_len of the absolute position
-    const int lo = max(split * split_len, first & ~(DEC_CHUNK - 1));
-    const int hi = min((split + 1) * split_len, kv_len);
-    const int32_t* table = block_tables + (int64_t)token_seq[t] * table_stride;
+    // A segment's block table entries: lane i keeps the entry of page lo / page_size + i (a segment
+    // spans at most 62 pages, so no chunk needs the table again).
+    auto first_of = [&](const int4& r) { return window > 0 && r.z - window + 1 > 0 ? r.z - window + 1 : 0; };
+    auto window_of = [&](const int4& r, int lo) {
+        const int page0 = lo / page_size;
+        return page0 + lane <= r.z / page_size ? block_tables[(int64_t)r.y * table_stride + page0 + lane] : -1;
+    };
+    auto load_q = [&](const int4& r, bf16x8* qf) {
+        // column `col` is query head kvh*G + col; lane group g holds channels [g*D/4, (g+1)*D/4)
+        const __bf16* qrow = q + (int64_t)r.x * q_stride + (int64_t)(kvh * G + (col < G ? col : 0)) * D + g * (D / 4);
+#pragma unroll
+        for (int c = 0; c < KP; ++c) qf[c] = *reinterpret_cast<const bf16x8*>(qrow + 8 * c);
+    };
 
-    // Q: column `col` is query head kvh*G + col; lane group g holds channels [g*D/4, (g+1)*D/4)
+    for (;;) {                                                           // over the wave's quotas: as a rule, one
+    // A quota's segments follow each other without a gap in the wave's loads: while it works on a
+    // segment, the record, the table entries and the query of the next are on their way, and the
+    // load that follows a segment's last chunk is the next segment's first chunk.  (After the
+    // quota's last segment the same segment is read once more and dropped.)
+    int4 rec = segments[2 * seg];
+    int lo = segments[2 * seg + 1].x, hi = segments[2 * seg + 1].y;
+    int table_window = window_of(rec, lo);
     bf16x8 qf[KP];
-    {
-        const __bf16* qrow = q + t * q_stride + (int64_t)(kvh * G + (col < G ? col : 0)) * D + g * (D / 4);
+    load_q(rec, qf);
+    bf16x8 ka_n[KP], kb_n[KP], vf_n[DT];
+    load_chunk<D>(lo, ka_n, kb_n, vf_n, k_cache, v_cache, table_window, lo / page_size, first_of(rec), rec.z + 1,
+                  num_kv_heads, kvh, page_size, row_key, col, g, error_flag);
+    int seg_next = min(seg + 1, seg_end - 1);
+    int4 rec_next = segments[2 * seg_next];
+    int2 range_next = *reinterpret_cast<const int2*>(&segments[2 * seg_next + 1]);
+
+    for (;;) {                                                           // over the quota's segments
+    const int64_t t = rec.x;
+    const int first = first_of(rec);
+    const int kv_len = rec.z + 1;
+    const int window_page0 = lo / page_size;
+    // the next segment: its table entries and its query (asked for now, used after this segment)
+    const int lo_next = range_next.x, hi_next = range_next.y;
+    const int first_next = first_of(rec_next);
+    const int table_window_next = window_of(rec_next, lo_next);
+    bf16x8 qf_next[KP];
+    load_q(rec_next, qf_next);
+    const int seg_after = min(seg_next + 1, seg_end - 1);
+    const int4 rec_after = segments[2 * seg_after];
+    const int2 range_after = *reinterpret_cast<const int2*>(&segments[2 * seg_after + 1]);
+    if (col >= G) {
 #pragma unroll
-        for (int c = 0; c < KP; ++c) {
-            bf16x8 v = *reinterpret_cast<const bf16x8*>(qrow + 8 * c);
-            if (col >= G) {
+        for (int c = 0; c < KP; ++c)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) v[e] = (__bf16)0.f;
-            }
-            qf[c] = v;
-        }
+            for (int e = 0; e < 8; ++e) qf[c][e] = (__bf16)0.f;
     }
 
     f32x4 acc[DT];
 #pragma unroll
     for (int i = 0; i < DT; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
-    // The loads of chunk i + 1 are issued before the products of chunk i, so that a wave always has
-    // a chunk (16 KiB at head_dim 128) in flight.
-    // Lane i of the wave keeps block table entry window_page0 + i: a split spans at most 64 pages
-    // (the launcher checks it), so no chunk needs the table again.
-    const int last_page = (kv_len - 1) / page_size;
-    const int window_page0 = lo / page_size;
-    const int table_window = window_page0 + lane <= last_page ? table[window_page0 + lane] : -1;
-    // The loads of the next chunk are issued, unconditionally, before the products of the current
-    // one (after the last chunk the same chunk is read once more and dropped): one path through the
-    // loop, so that the wait before the products covers exactly the current chunk's loads.
-    const int last_base = lo + ((hi - lo - 1) / DEC_CHUNK) * DEC_CHUNK;
-    bf16x8 ka_n[KP], kb_n[KP], vf_n[DT];
-    load_chunk<D>(lo, ka_n, kb_n, vf_n, k_cache, v_cache, table_window, window_page0, first, kv_len, num_kv_heads, kvh,
-                  page_size, row_key, col, g, error_flag);
+    // The loads of the chunk after are issued, unconditionally and on one path, before the products
+    // of the current chunk, so that a wave always has a chunk (16 KiB at head_dim 128) in flight and
+    // the wait before the products covers exactly the current chunk's loads.
     for (int base = lo; base < hi; base += DEC_CHUNK) {
         bf16x8 ka[KP], kb[KP], vf[DT];
 #pragma unroll
@@ -229,8 +269,13 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
         }
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) vf[dt] = vf_n[dt];
-        load_chunk<D>(min(base + DEC_CHUNK, last_base), ka_n, kb_n, vf_n, k_cache, v_cache, table_window, window_page0,
-                      first, kv_len, num_kv_heads, kvh, page_size, row_key, col, g, error_flag);
+        {
+            const bool last = base + DEC_CHUNK >= hi;                 // then the chunk after is the next segment's first
+            load_chunk<D>(last ? lo_next : base + DEC_CHUNK, ka_n, kb_n, vf_n, k_cache, v_cache,
+                          last ? table_window_next : table_window, last ? lo_next / page_size : window_page0,
+                          last ? first_next : first, last ? rec_next.z + 1 : kv_len, num_kv_heads, kvh,
+                          page_size, row_key, col, g, error_flag);
+        }
         if (base < first || base + DEC_CHUNK > kv_len) {
             // a chunk at an end of the visible range: what V holds outside the range may be anything
             const int key0 = base + 8 * g;
@@ -285,7 +330,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     // acc[dt][i] = O[head col][channel 16*dt + 4*g + i]
     if (col < G) {
         const int head = kvh * G + col;
-        if (splits_of_t == 1) {
+        if (rec.w == 1) {
             const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
             __bf16* orow = out + t * out_stride + (int64_t)head * D;
 #pragma unroll
@@ -293,7 +338,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
 #pragma unroll
                 for (int i = 0; i < 4; ++i) orow[16 * dt + 4 * g + i] = (__bf16)(acc[dt][i] * inv);
         } else {
-            const int64_t slot = (int64_t)flat * num_q_heads + head;
+            const int64_t slot = (int64_t)seg * num_q_heads + head;
             float* po = part_o + slot * D;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
@@ -304,14 +349,30 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
             }
         }
     }
+    if (seg + 1 >= seg_end) break;
+    seg = seg_next;
+    seg_next = seg_after;
+    rec = rec_next;
+    rec_next = rec_after;
+    range_next = range_after;
+    table_window = table_window_next;
+    lo = lo_next;
+    hi = hi_next;
+#pragma unroll
+    for (int c = 0; c < KP; ++c) qf[c] = qf_next[c];
+    }
+    quota += waves_per_head;
+    if (quota >= num_quotas) break;
+    seg = quota_first[quota];
+    seg_end = quota_first[quota + 1];
     }
 }
 
-// Merges the splits of one (token, head): o = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m); a
-// token with one split was written by the attention kernel itself.  One workgroup of four waves per
-// (token, head).  Every wave finds the maximum m over the splits, then takes every fourth group of
-// four splits (their loads overlap) and the four partial sums meet in LDS; the order of the sum
-// depends on the number of splits only.
+// Merges the segments of one (token, head): o = sum_s o_s e^(m_s - m) / sum_s l_s e^(m_s - m); a
+// token with one segment was written by the attention kernel itself.  One workgroup of four waves per
+// (token, head).  Every wave finds the maximum m over the segments, then takes every fourth group of
+// four segments (their loads overlap) and the four partial sums meet in LDS; the order of the sum
+// depends on the number of segments only.
 #define MERGE_WAVES 4
 __global__ void __launch_bounds__(MERGE_WAVES * NVA_WAVE)
 attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
@@ -321,7 +382,7 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
     __shared__ float l_s[MERGE_WAVES];
     const int64_t t = blockIdx.x;
     const int head = blockIdx.y, lane = threadIdx.x % NVA_WAVE, wave = threadIdx.x / NVA_WAVE;
-    const int s_lo = plan[2 + t], s_hi = plan[2 + t + 1] - 1;             // the token's splits, counted through
+    const int s_lo = plan[2 + t], s_hi = plan[2 + t + 1] - 1;             // the token's segments, counted through
     if (s_hi <= s_lo) return;
     auto slot_of = [&](int s) { return (int64_t)s * num_q_heads + head; };
     float m = -INFINITY;
@@ -333,7 +394,7 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
         float wj[4], v[4][4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const int s = min(s0 + j, s_hi);                              // a split past the end: read again, weight 0
+            const int s = min(s0 + j, s_hi);                              // a segment past the end: read again, weight 0
             const float ms = part_ml[slot_of(s) * 2];
             wj[j] = (s0 + j > s_hi || ms == -INFINITY) ? 0.f : __expf(ms - m);
             l += part_ml[slot_of(s) * 2 + 1] * wj[j];
@@ -370,51 +431,50 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
 }
 
 // What the decode attention of `tokens` single tokens needs when no request holds more than `longest`
-// keys: the bound of the splits of all tokens together, the number of persistent waves, and the size
-// of the plan (int32).  Partial results: max_total_splits * num_q_heads * (head_dim + 2) floats.
+// keys: the bound of the segments of all tokens together, the number of persistent waves (a multiple
+// of the kv heads), and the size of the plan (int32).  Partial results: max_segments * num_q_heads *
+// (head_dim + 2) floats.
 NVA_EXPORT int nva_attn_decode_plan_size_bf16(int longest, int64_t tokens, int num_kv_heads, int page_size,
-                                              int* max_total_splits, int* waves, int64_t* plan_ints) {
+                                              int* max_segments, int* waves, int64_t* plan_ints) {
     if (longest <= 0 || tokens <= 0 || tokens > DEC_MAX_TOKENS || num_kv_heads <= 0 || page_size <= 0 ||
-        !max_total_splits || !waves || !plan_ints)
+        !max_segments || !waves || !plan_ints)
         return nva_fail("attn_decode_plan_size: bad arguments (at most %d tokens a launch)", DEC_MAX_TOKENS);
-    const int64_t rows = tokens * num_kv_heads;
-    const int64_t wanted = (4 * DEC_RESIDENT_WAVES + rows - 1) / rows;
-    // sum of the tokens' counts <= total / len + 2 * tokens; len >= mean / wanted unless the page limit cuts it
-    const int cap = (62 * page_size) / DEC_CHUNK * DEC_CHUNK > DEC_CHUNK ? (62 * page_size) / DEC_CHUNK * DEC_CHUNK : DEC_CHUNK;
-    int64_t per_token = wanted;
-    if ((longest + cap - 1) / cap > per_token) per_token = (longest + cap - 1) / cap;
-    if (per_token > (longest + DEC_CHUNK - 1) / DEC_CHUNK) per_token = (longest + DEC_CHUNK - 1) / DEC_CHUNK;
-    const int64_t bound = tokens * (per_token + 2);
-    if (bound * num_kv_heads > 0x7fffffff || (longest + DEC_CHUNK - 1) / DEC_CHUNK > 0xffff)
-        return nva_fail("attn_decode_plan_size: too many splits");
-    *max_total_splits = (int)bound;
-    const int64_t items = bound * num_kv_heads;
-    *waves = (int)(items < DEC_RESIDENT_WAVES ? items : DEC_RESIDENT_WAVES);
-    *plan_ints = 2 + tokens + 1 + bound;
+    // a token sees at most longest / 32 + 2 chunks (a window may begin and end inside a chunk)
+    const int64_t chunks = tokens * ((int64_t)longest / DEC_CHUNK + 2);
+    int64_t per_head = DEC_RESIDENT_WAVES / num_kv_heads > 0 ? DEC_RESIDENT_WAVES / num_kv_heads : 1;
+    if (per_head > (chunks + 1) / 2) per_head = (chunks + 1) / 2;           // a quota has at least two chunks
+    const int64_t cap = decode_quota_cap(page_size);
+    const int64_t quotas = per_head > (chunks + cap - 1) / cap ? per_head : (chunks + cap - 1) / cap;
+    const int64_t bound = tokens + quotas;
+    if (bound * num_kv_heads > 0x7fffffff || per_head * num_kv_heads > 0x7fffffff)
+        return nva_fail("attn_decode_plan_size: too many segments");
+    *max_segments = (int)bound;
+    *waves = (int)(per_head * num_kv_heads);
+    *plan_ints = decode_plan_segments_at(tokens, bound) + 8 * bound;
     return 0;
 }
 
 // Makes the plan of a step (once per step and cache group; every layer's attention reads it).
-NVA_EXPORT int nva_attn_decode_plan_bf16(const int32_t* positions, int64_t tokens, int num_kv_heads, int page_size,
-                                         int window, int max_total_splits, int32_t* plan, int32_t* error_flag,
-                                         hipStream_t stream) {
-    if (!positions || !plan || tokens <= 0 || tokens > DEC_MAX_TOKENS || num_kv_heads <= 0 || page_size <= 0 ||
-        window < 0 || max_total_splits <= 0)
+// max_segments and waves from nva_attn_decode_plan_size for the same tokens, kv heads and page size.
+NVA_EXPORT int nva_attn_decode_plan_bf16(const int32_t* positions, const int32_t* token_seq, int64_t tokens,
+                                         int num_kv_heads, int page_size, int window, int max_segments, int waves,
+                                         int32_t* plan, int32_t* error_flag, hipStream_t stream) {
+    if (!positions || !token_seq || !plan || !nva_aligned(plan, 16) || tokens <= 0 || tokens > DEC_MAX_TOKENS ||
+        num_kv_heads <= 0 || page_size <= 0 || window < 0 || max_segments <= tokens || waves <= 0 || waves % num_kv_heads)
         return nva_fail("attn_decode_plan: bad arguments");
-    hipLaunchKernelGGL(attn_decode_plan_kernel, dim3(1), dim3(NVA_WAVE), 0, stream, positions, (int)tokens, num_kv_heads,
-                       page_size, window, max_total_splits, plan, error_flag);
+    hipLaunchKernelGGL(attn_decode_plan_kernel, dim3(1), dim3(NVA_WAVE), 0, stream, positions, token_seq, (int)tokens,
+                       page_size, window, max_segments, waves / num_kv_heads, plan, error_flag);
     return nva_check_launch("attn_decode_plan");
 }
 
 // Returns 1 (and leaves a message) for shapes this kernel does not take; the caller then uses the
 // general kernel.  plan: made by nva_attn_decode_plan for these tokens, kv heads, page size and
-// window; max_total_splits and waves from nva_attn_decode_plan_size.
+// window; max_segments and waves from nva_attn_decode_plan_size.
 NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride, float* scratch,
                                     const int32_t* plan, const void* k_cache, const void* v_cache,
-                                    const int32_t* block_tables, int table_stride, const int32_t* token_seq,
-                                    const int32_t* positions, int64_t tokens, int num_q_heads, int num_kv_heads,
-                                    int head_dim, int page_size, float scale, int window, int max_total_splits,
-                                    int waves, int32_t* error_flag, hipStream_t stream) {
+                                    const int32_t* block_tables, int table_stride, int64_t tokens, int num_q_heads,
+                                    int num_kv_heads, int head_dim, int page_size, float scale, int window,
+                                    int max_segments, int waves, int32_t* error_flag, hipStream_t stream) {
     if (tokens == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_decode: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
@@ -427,16 +487,17 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     if (tokens < 0 || tokens > DEC_MAX_TOKENS || num_q_heads > 65535)
         return nva_fail("attn_decode: %lld tokens (at most %d a launch) or %d heads exceed the grid", (long long)tokens,
                         DEC_MAX_TOKENS, num_q_heads);
-    if (max_total_splits <= 0 || waves <= 0 || window < 0 || table_stride <= 0 || !scratch || !plan)
-        return nva_fail("attn_decode: bad plan (%d splits, %d waves), window %d or no scratch", max_total_splits, waves,
+    if (max_segments <= tokens || waves <= 0 || waves % num_kv_heads || window < 0 || table_stride <= 0 || !scratch ||
+        !plan || !nva_aligned(plan, 16))
+        return nva_fail("attn_decode: bad plan (%d segments, %d waves), window %d or no scratch", max_segments, waves,
                         window);
     float* part_o = scratch;
-    float* part_ml = scratch + (int64_t)max_total_splits * num_q_heads * head_dim;
+    float* part_ml = scratch + (int64_t)max_segments * num_q_heads * head_dim;
 #define LAUNCH(DD)                                                                                              \
     hipLaunchKernelGGL(attn_decode_kernel<DD>, dim3((unsigned)waves), dim3(NVA_WAVE), 0, stream, (const __bf16*)q, \
                        q_stride, (__bf16*)out, out_stride, part_o, part_ml, plan, (const __bf16*)k_cache,         \
-                       (const __bf16*)v_cache, block_tables, table_stride, token_seq, positions, (int)tokens,     \
-                       num_q_heads, num_kv_heads, page_size, scale, window, error_flag)
+                       (const __bf16*)v_cache, block_tables, table_stride, (int)tokens, max_segments, num_q_heads,  \
+                       num_kv_heads, page_size, scale, window, error_flag)
     switch (head_dim) {
         case 32: LAUNCH(32); break;
         case 64: LAUNCH(64); break;

@@ -491,7 +491,7 @@ class HipKernels:
 
     def _attention_decode(self, q, qs, out, os_, k_cache, v_cache, tables, batch, n, num_heads, num_kv_heads,
                           head_dim, page_size, scale, window):
-        # The splits are planned on the device from the tokens' positions, once per step and (kv
+        # The work is shared out on the device from the tokens' positions, once per step and (kv
         # heads, window): the first layer that asks makes the plan, the others find it on the batch.
         # The library says how large the partial results may get for this many tokens of at most
         # max_kv_len keys, and how many persistent waves to launch.  At most 1024 tokens a launch.
@@ -507,15 +507,16 @@ class HipKernels:
                              c_i32(num_kv_heads), c_i32(page_size), ctypes.byref(bound), ctypes.byref(waves),
                              ctypes.byref(ints))
                 plan = torch.empty(ints.value, dtype=torch.int32, device=q.device)
-                library.call("attn_decode", "bf16", "nva_attn_decode_plan", _p(batch.positions[t0:t1]), c_i64(t1 - t0),
-                             c_i32(num_kv_heads), c_i32(page_size), c_i32(window or 0), c_i32(bound.value), _p(plan),
-                             _p(self.fault_flag), self._stream())
+                library.call("attn_decode", "bf16", "nva_attn_decode_plan", _p(batch.positions[t0:t1]),
+                             _p(batch.token_seq[t0:t1]), c_i64(t1 - t0),
+                             c_i32(num_kv_heads), c_i32(page_size), c_i32(window or 0), c_i32(bound.value),
+                             c_i32(waves.value), _p(plan), _p(self.fault_flag), self._stream())
                 plans[key] = (plan, bound.value, waves.value)
             plan, bound, waves = plans[key]
             scratch = torch.empty(bound * num_heads * (head_dim + 2), dtype=torch.float32, device=q.device)
             library.call("attn_decode", "bf16", "nva_attn_decode", _p(q[t0:t1]), c_i64(qs), _p(out[t0:t1]), c_i64(os_),
                          _p(scratch), _p(plan), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
-                         _p(batch.token_seq[t0:t1]), _p(batch.positions[t0:t1]), c_i64(t1 - t0), c_i32(num_heads),
+                         c_i64(t1 - t0), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
                          c_i32(bound), c_i32(waves), _p(self.fault_flag), self._stream())
 
