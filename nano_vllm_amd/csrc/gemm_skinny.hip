@@ -28,6 +28,8 @@ template <int MB> struct SkShape;
 template <> struct SkShape<1> { static constexpr int waves = 4; };
 template <> struct SkShape<2> { static constexpr int waves = 8; };
 template <> struct SkShape<4> { static constexpr int waves = 8; };
+// KW waves of a workgroup may share 16 rows of W and take every KW-th step of k each; their sums
+// meet in LDS.  That makes more and shorter waves without more partial sums in memory.
 
 __device__ __forceinline__ bf16x8 zero8() {
     bf16x8 z;
@@ -49,12 +51,11 @@ __device__ __forceinline__ bf16x8 zero8() {
 // the latency, so many short waves (a finer split of k) run faster than few long ones.  A chunk's
 // first loads are issued before its slice of x is staged.  Only a ragged last step (K % 256) moves
 // its offsets back into the row: what it reads beyond K meets zeros of x_s.
-template <int MB>
-__global__ void __launch_bounds__(SkShape<MB>::waves * NVA_WAVE)
+template <int MB, int WAVES, int KW>
+__global__ void __launch_bounds__(WAVES * NVA_WAVE)
 linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf16* __restrict__ w, int64_t w_stride,
                      float* __restrict__ partial, void* __restrict__ y, int64_t y_stride, int y_is_f32, int direct,
                      int M, int N, int K, int k_per_split, int chunk) {
-    constexpr int WAVES = SkShape<MB>::waves;
     constexpr int STEP = SK_KSTEP * SK_UNROLL;
     extern __shared__ __attribute__((aligned(16))) __bf16 x_s[];     // [M + 1][chunk + 8]
     const int wave = threadIdx.x / NVA_WAVE, lane = threadIdx.x % NVA_WAVE;
@@ -66,7 +67,8 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
 
     const bool gated = direct == 2;
     const int inner = N / 2;
-    const int tile = blockIdx.x * WAVES + wave;
+    const int tile = blockIdx.x * (WAVES / KW) + wave / KW;
+    const int ksub = wave % KW;
     const int n0 = gated ? tile * 8 : tile * 16;
     const bool active = n0 < (gated ? inner : N);     // idle waves still help to stage x
     const int w_row = gated ? min(n0 + (col & 7), inner - 1) + (col >= 8 ? inner : 0) : min(n0 + col, N - 1);
@@ -93,7 +95,7 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     for (int c_begin = k_begin; c_begin < k_end; c_begin += chunk) {
         const int c_end = min(k_end, c_begin + chunk);
         const int len = c_end - c_begin;
-        SK_LOAD_CLAMPED(c_begin);
+        SK_LOAD_CLAMPED(c_begin + ksub * STEP);
         // ---- stage x[0:M][c_begin:c_begin + chunk] and the zero row (zeros beyond c_end as well)
         __syncthreads();
         for (int idx = threadIdx.x; idx < (M + 1) * (chunk / 8); idx += WAVES * NVA_WAVE) {
@@ -104,25 +106,42 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
             *reinterpret_cast<bf16x8*>(&x_s[m * xs_stride + piece * 8]) = v;
         }
         __syncthreads();
-        if (!active) continue;
-        SK_PRODUCTS(0);
+        if (!active || ksub * STEP >= len) continue;
+        SK_PRODUCTS(ksub * STEP);
         const int full = len / STEP;
         const bf16x8* wp = reinterpret_cast<const bf16x8*>(wrow + c_begin + 8 * g);
-        int s = 1;
-        for (; s < full; ++s) {
+        int s = ksub + KW;
+        for (; s < full; s += KW) {
 #pragma unroll
             for (int u = 0; u < SK_UNROLL; ++u)
 #pragma unroll
                 for (int c = 0; c < 4; ++c) a[u][c] = wp[(s * STEP + u * SK_KSTEP + 32 * c) / 8];
             SK_PRODUCTS(s * STEP);
         }
-        if (s * STEP < len) {
+        if (s == full && s * STEP < len) {
             SK_LOAD_CLAMPED(c_begin + s * STEP);
             SK_PRODUCTS(s * STEP);
         }
     }
 #undef SK_LOAD_CLAMPED
 #undef SK_PRODUCTS
+    if (KW > 1) {
+        // the sums of the waves that share rows of W meet in LDS (x_s is done with), in a fixed order
+        f32x4* sums = reinterpret_cast<f32x4*>(x_s);                 // [WAVES][MB][lanes]
+        __syncthreads();
+        if (ksub != 0)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) sums[(wave * MB + b) * NVA_WAVE + lane] = acc[b];
+        __syncthreads();
+        if (ksub != 0) return;
+#pragma unroll
+        for (int o = 1; o < KW; ++o)
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const f32x4 v = sums[((wave + o) * MB + b) * NVA_WAVE + lane];
+                acc[b][0] += v[0]; acc[b][1] += v[1]; acc[b][2] += v[2]; acc[b][3] += v[3];
+            }
+    }
     if (!active) return;
     if (gated) {
         // acc[b][i] of lanes g < 2 is the gate of y[m = 16 * b + col][j = n0 + 4*g + i], the same register
@@ -203,13 +222,14 @@ linear_skinny_finish_kernel(const float* __restrict__ partial, int splits, const
     else ((__bf16*)y)[(int64_t)m * y_stride + j] = (__bf16)v;
 }
 
-// splits: how many ranges k is cut into (>= 1); scratch must hold splits * M * N floats when
+// waves_per_tile: 1, 2 or 4 waves of a workgroup share 16 rows of W and split the k range between
+// them (pays for very few rows of x).  splits: how many ranges k is cut into (>= 1); scratch must hold splits * M * N floats when
 // splits > 1 or a bias, swiglu or defer_finish is asked for.  splits_used receives the number of
 // ranges really used (k per range is rounded up to a multiple of 256).  Returns 1 for shapes this kernel does not take.
 NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
                                       const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
-                                      float* scratch, int splits, int defer_finish, int64_t M, int64_t N,
-                                      int64_t K, int* splits_used, hipStream_t stream) {
+                                      float* scratch, int splits, int waves_per_tile, int defer_finish, int64_t M,
+                                      int64_t N, int64_t K, int* splits_used, hipStream_t stream) {
     if (M == 0 || N == 0) return 0;
     if (M < 0 || M > SK_MAX_ROWS || K % 8 || K <= 0 || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
         nva_fail("linear_skinny: needs 1..%d rows, K %% 8 == 0 and 16-byte aligned rows (M=%lld K=%lld)", SK_MAX_ROWS,
@@ -217,6 +237,8 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
         return 1;
     }
     if (N > 0x7fffffff || K > 0x7fffffff || splits < 1 || splits > 65535) return nva_fail("linear_skinny: bad sizes");
+    if (waves_per_tile != 1 && waves_per_tile != 2 && waves_per_tile != 4)
+        return nva_fail("linear_skinny: 1, 2 or 4 waves share rows of W, not %d", waves_per_tile);
     if (swiglu && (N % 2)) return nva_fail("linear_skinny: the gated form needs an even number of weight rows");
     const int direct = splits == 1 && !bias && !defer_finish ? (swiglu ? 2 : 1) : 0;
     if (!direct && !scratch) return nva_fail("linear_skinny: this call needs scratch memory");
@@ -228,18 +250,26 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     int chunk = (36864 / (2 * ((int)M + 1)) - 8) / 256 * 256;
     chunk = chunk < 256 ? 256 : chunk > 2048 ? 2048 : chunk;
     if (chunk > kps) chunk = kps;
-    const size_t lds = (size_t)(M + 1) * (chunk + 8) * sizeof(__bf16);
-#define LAUNCH(MB)                                                                                                     \
+    size_t lds = (size_t)(M + 1) * (chunk + 8) * sizeof(__bf16);
+#define LAUNCH(MB, KW)                                                                                                 \
     do {                                                                                                               \
-        constexpr int waves = SkShape<MB>::waves;                                                                      \
-        dim3 grid((unsigned)((tiles + waves - 1) / waves), (unsigned)real_splits);                                     \
-        hipLaunchKernelGGL(linear_skinny_kernel<MB>, grid, dim3(waves * NVA_WAVE), lds, stream, (const __bf16*)x,      \
-                           x_stride, (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32, direct, (int)M,       \
-                           (int)N, (int)K, kps, chunk);                                                                \
+        constexpr int waves = SkShape<MB>::waves, per_wg = waves / KW;                                                 \
+        if (KW > 1 && lds < (size_t)waves * MB * NVA_WAVE * sizeof(f32x4)) lds = (size_t)waves * MB * NVA_WAVE * sizeof(f32x4); \
+        dim3 grid((unsigned)((tiles + per_wg - 1) / per_wg), (unsigned)real_splits);                                   \
+        hipLaunchKernelGGL((linear_skinny_kernel<MB, waves, KW>), grid, dim3(waves * NVA_WAVE), lds, stream,                  \
+                           (const __bf16*)x, x_stride, (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32,     \
+                           direct, (int)M, (int)N, (int)K, kps, chunk);                                                \
     } while (0)
-    if (M <= 16) LAUNCH(1);
-    else if (M <= 32) LAUNCH(2);
-    else LAUNCH(4);
+#define LAUNCH_KW(MB)                                                                                                  \
+    do {                                                                                                               \
+        if (waves_per_tile == 1) LAUNCH(MB, 1);                                                                        \
+        else if (waves_per_tile == 2) LAUNCH(MB, 2);                                                                   \
+        else LAUNCH(MB, 4);                                                                                            \
+    } while (0)
+    if (M <= 16) LAUNCH_KW(1);
+    else if (M <= 32) LAUNCH_KW(2);
+    else LAUNCH_KW(4);
+#undef LAUNCH_KW
 #undef LAUNCH
     if (splits_used) *splits_used = real_splits;
     int rc = nva_check_launch("linear_skinny");

@@ -170,7 +170,7 @@ struct AdvanceGroups {
 
 __global__ void advance_decode_kernel(int32_t* __restrict__ input_ids, int32_t* __restrict__ positions,
                                       int32_t* __restrict__ kv_lens, int32_t* __restrict__ starts,
-                                      int32_t* __restrict__ max_kv, const int32_t* __restrict__ sampled,
+                                      const int32_t* __restrict__ sampled,
                                       int32_t* __restrict__ out_row, int n_real, int n_total, int page_size,
                                       AdvanceGroups groups, int num_groups, int32_t* error_flag) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -194,11 +194,10 @@ __global__ void advance_decode_kernel(int32_t* __restrict__ input_ids, int32_t* 
         }
         groups.slots[g][i] = slot;
     }
-    if (i == 0) max_kv[0] += 1;
 }
 
 NVA_EXPORT int nva_advance_decode(int32_t* input_ids, int32_t* positions, int32_t* kv_lens, int32_t* starts,
-                                  int32_t* max_kv, const int32_t* sampled, int32_t* out_row, int n_real, int n_total,
+                                  const int32_t* sampled, int32_t* out_row, int n_real, int n_total,
                                   int page_size, int num_groups, int32_t* const* slots, const int32_t* const* tables,
                                   const int* widths, int32_t* error_flag, hipStream_t stream) {
     if (n_real <= 0 || n_total < n_real || page_size <= 0 || num_groups < 0 || num_groups > ADVANCE_MAX_GROUPS)
@@ -210,7 +209,7 @@ NVA_EXPORT int nva_advance_decode(int32_t* input_ids, int32_t* positions, int32_
         groups.width[g] = widths[g];
     }
     hipLaunchKernelGGL(advance_decode_kernel, dim3((unsigned)((n_total + 255) / 256)), dim3(256), 0, stream, input_ids,
-                       positions, kv_lens, starts, max_kv, sampled, out_row, n_real, n_total, page_size, groups, num_groups,
+                       positions, kv_lens, starts, sampled, out_row, n_real, n_total, page_size, groups, num_groups,
                        error_flag);
     return nva_check_launch("advance_decode");
 }

@@ -43,7 +43,6 @@ class StepBatch:
     kv_lens: torch.Tensor            # int32 [S] keys each request sees = start + its tokens
     seq_starts: torch.Tensor         # int32 [S] tokens each request had in the cache before
     state_slots: torch.Tensor        # int32 [S]
-    max_kv_dev: torch.Tensor         # int32 [1]: max(kv_lens), for kernels of a replayed launch
     logits_rows: Optional[torch.Tensor]   # int32 [R] flat token indices, in the caller's order
     prefill_tiles: Optional[torch.Tensor]  # int32 [tiles, 2]: (request, 32-row tile) of the portions, most keys first
     groups: List[GroupBatch]
@@ -53,7 +52,6 @@ class StepBatch:
     q_lens: List[int] = field(default_factory=list)
     starts: List[int] = field(default_factory=list)
     requests: List[Hashable] = field(default_factory=list)
-    lengths_vary: bool = False       # a captured launch: max_kv_len is a bound of the steps it is replayed for
     step_cache: dict = field(default_factory=dict)   # emptied by the model at the start of every pass
 
 
@@ -164,7 +162,7 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
             raise ValueError(f"a block table of {max(widths)} pages exceeds the fixed width {table_width}")
         widths = [table_width] * num_groups
     tile_order = prefill_tile_order(q_lens, starts, num_decode)
-    scalars = cu + kv_lens + starts + state_slots + [max(kv_lens)] + rows + tile_order
+    scalars = cu + kv_lens + starts + state_slots + rows + tile_order
     if num_decode == S:                              # decoded tokens only: one list, one conversion
         flat: List[int] = one_ids + one_pos + list(range(S)) + scalars
         for g in range(num_groups):
@@ -202,7 +200,7 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
         return out
 
     b_ids, b_pos, b_seq = take(T), take(T), take(T)
-    b_cu, b_kv, b_starts, b_slots, b_max_kv = take(S + 1), take(S), take(S), take(S), take(1)
+    b_cu, b_kv, b_starts, b_slots = take(S + 1), take(S), take(S), take(S)
     b_rows = take(len(rows)) if rows else None
     b_tiles = take(len(tile_order)).view(-1, 2) if tile_order else None
     groups = []
@@ -213,6 +211,6 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
     return StepBatch(
         num_tokens=T, num_seqs=S, num_decode=num_decode, prefill_tiles=b_tiles,
         input_ids=b_ids, positions=b_pos, token_seq=b_seq, cu_seqlens_q=b_cu, kv_lens=b_kv,
-        seq_starts=b_starts, state_slots=b_slots, max_kv_dev=b_max_kv, logits_rows=b_rows, groups=groups,
+        seq_starts=b_starts, state_slots=b_slots, logits_rows=b_rows, groups=groups,
         max_q_len=max(q_lens), max_kv_len=max(kv_lens), q_lens=q_lens, starts=starts,
         requests=[entries[i].request for i in order])

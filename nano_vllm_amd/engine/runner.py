@@ -106,12 +106,11 @@ class ModelRunner:
             # the flat layout of size_b single tokens with every logit wanted and tables of fixed width
             num_groups = len(self.groups)
             b = size_b
-            size = 3 * b + (b + 1) + 3 * b + 1 + b + num_groups * (b + b * self._graph_table_width)
+            size = 3 * b + (b + 1) + 3 * b + b + num_groups * (b + b * self._graph_table_width)
             static = torch.zeros(size, dtype=torch.int32, device=self.device)
             batch = build_batch(entries, self.cache, self.page_size, vocab, self.device,
                                 table_width=self._graph_table_width, static=static, pad_to=size_b)
             batch.max_kv_len = self._graph_max_len        # launch shapes must cover every later step
-            batch.lengths_vary = True
             side = torch.cuda.Stream(self.device)
             side.wait_stream(torch.cuda.current_stream(self.device))
             with torch.cuda.stream(side):                 # what is set up lazily is set up outside the capture

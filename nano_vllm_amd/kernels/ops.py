@@ -121,6 +121,7 @@ class HipKernels:
         self.own_matmul_rows = 16           # bfloat16 products with more rows go to the library ...
         self.skinny_max_rows = 64           # ... unless the weight is small (see _own_rows); the kernel's limit
         self.small_weight_bytes = 64 << 20
+        self.skinny_waves_per_tile = 0      # waves of a workgroup that share rows of the weight and split k; 0: by rows of x
         self.skinny_target_waves = 4096     # the k range of a few-row product is split until this many waves run
         self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
@@ -302,8 +303,11 @@ class HipKernels:
         tiles = (n + 15) // 16
         # many rows of x: the partial sums weigh more, and the waves do more work each
         target = self.skinny_target_waves if m <= 16 else self.skinny_target_waves // 2
-        splits = max(1, min((target + tiles - 1) // tiles, k // 256))
-        if swiglu and bias is None and 2 * tiles >= target:
+        # few rows of x: staging them costs little, and four waves that share rows of the weight and
+        # split k between them inside the workgroup leave fewer partial sums to add
+        kw = self.skinny_waves_per_tile or (4 if m <= 4 else 1)
+        splits = max(1, min((target + tiles * kw - 1) // (tiles * kw), k // 256))
+        if swiglu and bias is None and 2 * tiles * kw >= target:
             splits = 1          # wide enough without a split of k: the gating happens in the product kernel
         if defer and splits == 1:
             defer = False
@@ -314,7 +318,7 @@ class HipKernels:
         used = ctypes.c_int(0)
         library.call("gemm_skinny", "bf16", "nva_linear_skinny", _p(x), c_i64(xs), _p(weight), c_i64(ws),
                      None if defer else _p(bias), _p(out), c_i64(os_), c_i32(1 if out_float32 else 0),
-                     c_i32(1 if swiglu else 0), _p(scratch), c_i32(splits), c_i32(1 if defer else 0), c_i64(m), c_i64(n),
+                     c_i32(1 if swiglu else 0), _p(scratch), c_i32(splits), c_i32(kw), c_i32(1 if defer else 0), c_i64(m), c_i64(n),
                      c_i64(k), ctypes.byref(used), self._stream())
         if defer:
             return SplitSum(self, scratch, used.value, m, n, bias)
@@ -562,5 +566,5 @@ class HipKernels:
         slots = ptr(*[g.slot_mapping.data_ptr() for g in groups])
         tables = ptr(*[g.block_tables.data_ptr() for g in groups])
         library.call("sample", None, "nva_advance_decode", _p(batch.input_ids), _p(batch.positions), _p(batch.kv_lens),
-                     _p(batch.seq_starts), _p(batch.max_kv_dev), _p(sampled), _p(out_row), c_i32(n_real), c_i32(n_total),
+                     _p(batch.seq_starts), _p(sampled), _p(out_row), c_i32(n_real), c_i32(n_total),
                      c_i32(page_size), c_i32(len(groups)), slots, tables, widths, _p(self.fault_flag), self._stream())

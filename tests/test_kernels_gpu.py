@@ -138,7 +138,8 @@ def test_linear_bfloat16(hip, ref, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (8, 6144, 4096), (64, 320, 12288), (17, 1000, 264), (33, 24, 8),
-                                   (5, 130, 72), (48, 40000, 1288), (20, 40004, 2304), (64, 4096, 4096)])
+                                   (5, 130, 72), (48, 40000, 1288), (20, 40004, 2304), (64, 4096, 4096),
+                                   (2, 1000, 1288), (4, 40004, 2304), (3, 130, 72), (4, 4096, 12288)])
 def test_linear_bfloat16_few_rows_streams_the_weights(hip, ref, m, n, k):
     """The decode-step product (few rows, k split over workgroups) against a double product."""
     x, w = _rand((m, k), torch.bfloat16, 21), _rand((n, k), torch.bfloat16, 22, 0.05)
@@ -154,7 +155,7 @@ def test_linear_bfloat16_few_rows_streams_the_weights(hip, ref, m, n, k):
 
 
 @pytest.mark.parametrize("m,inner,k", [(1, 12288, 4096), (8, 200, 96), (64, 160, 256), (100, 64, 128), (5, 8196, 264),
-                                       (40, 9004, 1288), (16, 12288, 4096)])
+                                       (40, 9004, 1288), (16, 12288, 4096), (2, 8196, 264), (4, 9004, 1288), (3, 200, 96)])
 def test_linear_silu_mul(hip, ref, m, inner, k):
     x, w = _rand((m, k), torch.bfloat16, 24), _rand((2 * inner, k), torch.bfloat16, 25, 0.1)
     _close(hip[torch.bfloat16].linear_silu_mul(x, w), ref.linear_silu_mul(x, w), torch.bfloat16)
