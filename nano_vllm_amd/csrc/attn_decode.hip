@@ -238,14 +238,23 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     const int kv_len = rec.z + 1;
     const int window_page0 = lo / page_size;
     // the next segment: its table entries and its query (asked for now, used after this segment)
+    // (after the quota's last segment there is none: the loads past its end then all meet the
+    // segment's last key, which is visible and whose page the wave's table entries hold)
+    const bool more = seg + 1 < seg_end;
     const int lo_next = range_next.x, hi_next = range_next.y;
-    const int first_next = first_of(rec_next);
-    const int table_window_next = window_of(rec_next, lo_next);
+    const int first_next = more ? first_of(rec_next) : hi_next - 1;
+    const int kv_len_next = more ? rec_next.z + 1 : hi_next;
+    int table_window_next = table_window;
     bf16x8 qf_next[KP];
-    load_q(rec_next, qf_next);
+    int4 rec_after = rec_next;
+    int2 range_after = range_next;
     const int seg_after = min(seg_next + 1, seg_end - 1);
-    const int4 rec_after = segments[2 * seg_after];
-    const int2 range_after = *reinterpret_cast<const int2*>(&segments[2 * seg_after + 1]);
+    if (more) {
+        table_window_next = window_of(rec_next, lo_next);
+        load_q(rec_next, qf_next);
+        rec_after = segments[2 * seg_after];
+        range_after = *reinterpret_cast<const int2*>(&segments[2 * seg_after + 1]);
+    }
     if (col >= G) {
 #pragma unroll
         for (int c = 0; c < KP; ++c)
@@ -273,7 +282,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
             const bool last = base + DEC_CHUNK >= hi;                 // then the chunk after is the next segment's first
             load_chunk<D>(last ? lo_next : base + DEC_CHUNK, ka_n, kb_n, vf_n, k_cache, v_cache,
                           last ? table_window_next : table_window, last ? lo_next / page_size : window_page0,
-                          last ? first_next : first, last ? rec_next.z + 1 : kv_len, num_kv_heads, kvh,
+                          last ? first_next : first, last ? kv_len_next : kv_len, num_kv_heads, kvh,
                           page_size, row_key, col, g, error_flag);
         }
         if (base < first || base + DEC_CHUNK > kv_len) {
@@ -349,7 +358,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
             }
         }
     }
-    if (seg + 1 >= seg_end) break;
+    if (!more) break;
     seg = seg_next;
     seg_next = seg_after;
     rec = rec_next;

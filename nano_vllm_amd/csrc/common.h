@@ -156,7 +156,7 @@ __device__ __forceinline__ void partial_value8(const PartialInput& p, int64_t ro
     const float* q = p.sums + row * width + i;
 #pragma unroll
     for (int e = 0; e < 8; ++e) out[e] = 0.f;
-#pragma unroll 4
+#pragma unroll 8
     for (int s = 0; s < p.splits; ++s) {
         float v[8];
         load8(q + s * p.split_stride, v);

@@ -16,7 +16,7 @@
 #define NORM_KEEP 2
 
 template <typename T, bool ADD, bool VEC>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 rms_norm_kernel(const T* x, int64_t x_stride, PartialInput part, T* residual, int64_t r_stride,
                 const void* __restrict__ weight, int w_is_f32, T* y, int64_t y_stride,
                 int width, float eps) {
@@ -132,7 +132,8 @@ static int launch(const elem_t* x, int64_t x_stride, PartialInput part, elem_t* 
                      nva_aligned(y, vec_bytes) &&
                      (!ADD || nva_aligned(residual, vec_bytes)) &&
                      nva_aligned(weight, w_is_f32 ? 32 : vec_bytes);
-    const int threads = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
+    // few wide rows: one vector of 8 per thread, so that a row of partial sums is read in one round of loads
+    const int threads = width >= 4096 && rows <= 256 ? 512 : width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
     if (vec)
         hipLaunchKernelGGL((rms_norm_kernel<elem_t, ADD, true>), dim3((unsigned)rows), dim3(threads), 0, stream,
                            x, x_stride, part, residual, r_stride, weight, w_is_f32, y, y_stride, width, eps);
