@@ -13,6 +13,7 @@
 // Requires K % 8 == 0 and 16-byte aligned rows; the launcher refuses anything else and the caller
 // uses the library product or the tiled kernel.
 #include "common.h"
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -193,6 +194,167 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     }
 }
 
+// The same product for more rows of x (up to 128), where the slice of x no longer fits LDS for a
+// long range of k and the reads of x from LDS weigh as much as the products.  A workgroup of four
+// waves takes 16 * RT rows of W per wave and walks its k range in chunks of 128: the chunk of x
+// lies in LDS twice (the next one is fetched into registers during the products and written to
+// the other half, one barrier per chunk), every fragment of x read from LDS feeds RT products, and
+// each 16-byte piece of W is asked for again, one chunk ahead, as soon as its products are issued.
+// direct and the layout of the results: as above.
+#define MD_KC 128
+#define MD_XS (MD_KC + 8)
+template <int MB, int RT>
+__global__ void __launch_bounds__(4 * NVA_WAVE) __attribute__((amdgpu_waves_per_eu(2)))
+linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf16* __restrict__ w, int64_t w_stride,
+                     float* __restrict__ partial, void* __restrict__ y, int64_t y_stride, int y_is_f32, int direct,
+                     int M, int N, int K, int k_per_split) {
+    constexpr int ROWS = 16 * MB + 1;                                 // the last row stays zero when M = 16 * MB
+    extern __shared__ __attribute__((aligned(16))) __bf16 x_s[];      // [2][ROWS][MD_XS]
+    const int wave = threadIdx.x / NVA_WAVE, lane = threadIdx.x % NVA_WAVE;
+    const int col = lane & 15, g = lane >> 4;
+    const int split = blockIdx.y;
+    const int k_begin = split * k_per_split;
+    const int k_end = min(K, k_begin + k_per_split);
+    const int chunks = (k_end - k_begin + MD_KC - 1) / MD_KC;
+    const bool gated = direct == 2;
+    const int inner = N / 2;
+    const int per_tile = gated ? 8 : 16;
+    const int tile0 = (blockIdx.x * 4 + wave) * RT;
+    const int k_last = K - 8;
+
+    const __bf16* wrow[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int n0 = (tile0 + rt) * per_tile;
+        const int w_row = gated ? min(n0 + (col & 7), inner - 1) + (col >= 8 ? inner : 0) : min(n0 + col, N - 1);
+        wrow[rt] = w + (int64_t)w_row * w_stride + 8 * g;
+    }
+    int xoff[MB];
+    f32x4 acc[RT][MB];
+#pragma unroll
+    for (int b = 0; b < MB; ++b) {
+        xoff[b] = min(col + 16 * b, M) * MD_XS + 8 * g;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt) acc[rt][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    // staging: thread t moves the 16-byte piece t % 16 of rows t / 16 + 16 * j
+    const int s_row = threadIdx.x / 16, s_piece = threadIdx.x % 16;
+    bf16x8 xr[MB];
+    // (every load of the loop is unconditional, from an address moved into the operand where it
+    // would lie outside, and what must be zero is made zero when it is written to LDS: a branch
+    // around a load makes the compiler wait for all loads in flight at every turn)
+    auto fetch_x = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < MB; ++j)
+            xr[j] = *reinterpret_cast<const bf16x8*>(x + (int64_t)min(s_row + 16 * j, M - 1) * x_stride +
+                                                     min(k0 + 8 * s_piece, k_last));
+    };
+    auto store_x = [&](int buf, int k0) {
+        const bool k_ok = k0 + 8 * s_piece < k_end;
+#pragma unroll
+        for (int j = 0; j < MB; ++j)
+            *reinterpret_cast<bf16x8*>(&x_s[(buf * ROWS + s_row + 16 * j) * MD_XS + 8 * s_piece]) =
+                k_ok && s_row + 16 * j < M ? xr[j] : zero8();
+    };
+    // W of two chunks is in registers or on its way at any time (16 KiB per wave with RT = 2): with
+    // so few waves per CU, less in flight does not cover the memory's latency
+    // Workgroups walk their chunks in rotated order, each from another start: at one k the rows of
+    // x (a power of two apart, as a rule) lie in few channels of the L2, and workgroups that all
+    // fetch the same chunk at the same time queue up there.
+    const int rot = (blockIdx.x * 5 + blockIdx.y) % chunks;
+    // (past the last chunk: K, from where every load is moved back to the rows' last pieces)
+    auto k_of = [&](int c) { return c < chunks ? k_begin + (c + rot) % chunks * MD_KC : K; };
+    bf16x8 a[2][RT][4];
+    fetch_x(k_of(0));
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+                a[h][rt][c] = *reinterpret_cast<const bf16x8*>(wrow[rt] + min(k_of(h) + 32 * c, k_last - 8 * g));
+    if (threadIdx.x < 2 * (MD_XS / 8)) {                              // the row beyond the staged ones, in both halves
+        const int buf = threadIdx.x / (MD_XS / 8), piece = threadIdx.x % (MD_XS / 8);
+        *reinterpret_cast<bf16x8*>(&x_s[(buf * ROWS + ROWS - 1) * MD_XS + 8 * piece]) = zero8();
+    }
+    store_x(0, k_of(0));
+    __syncthreads();
+    auto chunk = [&](int c, auto half) {
+        constexpr int H = decltype(half)::value;                      // the half of x_s and of `a` this chunk uses
+        const int k_next = k_of(c + 1), k_ahead = k_of(c + 2);
+        fetch_x(k_next);
+        const __bf16* xb = x_s + H * ROWS * MD_XS;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const bf16x8 frag = *reinterpret_cast<const bf16x8*>(xb + xoff[b] + 32 * p);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    acc[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[H][rt][p], frag, acc[rt][b], 0, 0, 0);
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)      // past the last chunk all lanes read one piece of the first row
+                a[H][rt][p] = *reinterpret_cast<const bf16x8*>((c + 2 < chunks ? wrow[rt] : w + 8 * g) + min(k_ahead + 32 * p, k_last - 8 * g));
+        }
+        store_x(H ^ 1, k_next);                                      // after the last chunk: written, never read
+        __syncthreads();
+    };
+    for (int c = 0; c < chunks; c += 2) {
+        chunk(c, std::integral_constant<int, 0>());
+        if (c + 1 < chunks) chunk(c + 1, std::integral_constant<int, 1>());
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int n0 = (tile0 + rt) * per_tile;
+        if (n0 >= (gated ? inner : N)) continue;
+        if (gated) {
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                const int m = 16 * b + col;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float up = (float)(__bf16)__shfl(acc[rt][b][i], (lane + 32) % NVA_WAVE, NVA_WAVE);
+                    const float gate = (float)(__bf16)acc[rt][b][i];
+                    const int j = n0 + 4 * g + i;
+                    if (g < 2 && m < M && j < inner) {
+                        const float v = gate / (1.f + __expf(-gate)) * up;
+                        if (y_is_f32) ((float*)y)[(int64_t)m * y_stride + j] = v;
+                        else ((__bf16*)y)[(int64_t)m * y_stride + j] = (__bf16)v;
+                    }
+                }
+            }
+            continue;
+        }
+        const int n = n0 + 4 * g;
+#pragma unroll
+        for (int b = 0; b < MB; ++b) {
+            const int m = 16 * b + col;
+            if (m >= M) continue;
+            if (!direct) {
+                float* p = partial + ((int64_t)split * M + m) * N + n;
+                if (n + 3 < N && (N % 4) == 0) {
+                    *reinterpret_cast<f32x4*>(p) = acc[rt][b];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (n + i < N) p[i] = acc[rt][b][i];
+                }
+            } else if (y_is_f32) {
+                float* p = (float*)y + (int64_t)m * y_stride + n;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < N) p[i] = acc[rt][b][i];
+            } else {
+                __bf16* p = (__bf16*)y + (int64_t)m * y_stride + n;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < N) p[i] = (__bf16)acc[rt][b][i];
+            }
+        }
+    }
+}
+
 // y[m][n] = sum over splits of partial[s][m][n] (+ bias[n]); with swiglu, N is the width of the
 // partials (2 * inner) and y[m][j] = silu(sum_gate[j]) * sum_up[j], j < inner.
 __global__ void __launch_bounds__(256)
@@ -274,6 +436,58 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     if (splits_used) *splits_used = real_splits;
     int rc = nva_check_launch("linear_skinny");
     // deferred: the partial sums [real_splits][M][N] stay in scratch for a kernel that consumes them
+    if (rc || direct || defer_finish) return rc;
+    const int64_t outs = M * (swiglu ? N / 2 : N);
+    hipLaunchKernelGGL(linear_skinny_finish_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, stream, scratch,
+                       real_splits, (const __bf16*)bias, y, y_stride, y_is_f32, swiglu, (int)M, (int)N);
+    return nva_check_launch("linear_skinny_finish");
+}
+
+// The kernel for up to 128 rows of x.  row_tiles: 1 or 2 blocks of 16 rows of W per wave.  The other
+// arguments as for nva_linear_skinny; k per range is rounded up to a multiple of 128.
+NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
+                                      const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
+                                      float* scratch, int splits, int row_tiles, int defer_finish, int64_t M,
+                                      int64_t N, int64_t K, int* splits_used, hipStream_t stream) {
+    if (M == 0 || N == 0) return 0;
+    if (M < 0 || M > 128 || K % 8 || K <= 0 || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
+        nva_fail("linear_medium: needs 1..128 rows, K %% 8 == 0 and 16-byte aligned rows (M=%lld K=%lld)", (long long)M,
+                 (long long)K);
+        return 1;
+    }
+    if (N > 0x7fffffff || K > 0x7fffffff || splits < 1 || splits > 65535) return nva_fail("linear_medium: bad sizes");
+    if (row_tiles != 1 && row_tiles != 2) return nva_fail("linear_medium: 1 or 2 row tiles per wave, not %d", row_tiles);
+    if (swiglu && (N % 2)) return nva_fail("linear_medium: the gated form needs an even number of weight rows");
+    const int direct = splits == 1 && !bias && !defer_finish ? (swiglu ? 2 : 1) : 0;
+    if (!direct && !scratch) return nva_fail("linear_medium: this call needs scratch memory");
+    int kps = (int)((K + splits - 1) / splits);
+    kps = (kps + MD_KC - 1) / MD_KC * MD_KC;
+    const int real_splits = (int)((K + kps - 1) / kps);
+    const int64_t tiles = direct == 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
+    const int mb = (int)((M + 15) / 16 + 1) / 2 * 2;                   // instances for 2, 4, 6, 8 blocks of 16 rows
+    const size_t lds = (size_t)2 * (16 * mb + 1) * MD_XS * sizeof(__bf16);
+#define LAUNCH(MB, RT)                                                                                                 \
+    do {                                                                                                               \
+        dim3 grid((unsigned)((tiles + 4 * RT - 1) / (4 * RT)), (unsigned)real_splits);                                 \
+        hipLaunchKernelGGL((linear_medium_kernel<MB, RT>), grid, dim3(4 * NVA_WAVE), lds, stream, (const __bf16*)x,    \
+                           x_stride, (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32, direct, (int)M,       \
+                           (int)N, (int)K, kps);                                                                       \
+    } while (0)
+#define LAUNCH_RT(MB)                                                                                                  \
+    do {                                                                                                               \
+        if (row_tiles == 1) LAUNCH(MB, 1);                                                                             \
+        else LAUNCH(MB, 2);                                                                                            \
+    } while (0)
+    switch (mb) {
+        case 2: LAUNCH_RT(2); break;
+        case 4: LAUNCH_RT(4); break;
+        case 6: LAUNCH_RT(6); break;
+        default: LAUNCH_RT(8); break;
+    }
+#undef LAUNCH_RT
+#undef LAUNCH
+    if (splits_used) *splits_used = real_splits;
+    int rc = nva_check_launch("linear_medium");
     if (rc || direct || defer_finish) return rc;
     const int64_t outs = M * (swiglu ? N / 2 : N);
     hipLaunchKernelGGL(linear_skinny_finish_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, stream, scratch,

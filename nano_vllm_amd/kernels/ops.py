@@ -121,6 +121,10 @@ class HipKernels:
         self.own_matmul_rows = 16           # bfloat16 products with more rows go to the library ...
         self.skinny_max_rows = 64           # ... unless the weight is small (see _own_rows); the kernel's limit
         self.small_weight_bytes = 64 << 20
+        self.medium_max_rows = 128          # rows of x the kernel for medium row counts takes
+        self.medium_max_weight_rows = 8192  # and the widest weight it is used for
+        self.medium_row_tiles = 2           # blocks of 16 weight rows per wave in the kernel for up to 128 rows
+        self.medium_target_workgroups = 256 # its k range is split until about this many workgroups run (one per CU)
         self.skinny_waves_per_tile = 0      # waves of a workgroup that share rows of the weight and split k; 0: by rows of x
         self.skinny_target_waves = 4096     # the k range of a few-row product is split until this many waves run
         self.fuse_split_sums = True         # False: every product is finished by its own pass
@@ -253,15 +257,19 @@ class HipKernels:
             raise KernelError("linear: bias does not fit")
         out_dtype = torch.float32 if out_float32 else x.dtype
         if x.dtype == torch.bfloat16 and self._skinny_takes(x, xs, weight, ws, k):
-            own = 0 < m <= self._own_rows(n, k)
+            own = self._own_kernel(m, n, k)
+            run = self._linear_medium if own == "medium" else self._linear_skinny
             if deferred and own and not out_float32 and out is None and self.fuse_split_sums:
-                return self._linear_skinny(x, xs, weight, ws, bias, None, 0, False, False, m, n, k, defer=True)
+                return run(x, xs, weight, ws, bias, None, 0, False, False, m, n, k, defer=True)
             if own or out_float32:
                 if out is None:
                     out = torch.empty((m, n), dtype=out_dtype, device=x.device)
                 om, on, os_ = _rows2d(out, "linear output")
                 if (om, on) != (m, n) or out.dtype != out_dtype:
                     raise KernelError("linear: output does not match")
+                if own == "medium":
+                    self._linear_medium(x, xs, weight, ws, bias, out, os_, out_float32, False, m, n, k)
+                    return out
                 rows = self.skinny_max_rows      # more rows (logits of many places): that many at a time
                 for r0 in range(0, m, rows):
                     r1 = min(m, r0 + rows)
@@ -283,14 +291,23 @@ class HipKernels:
                      c_i64(m), c_i64(n), c_i64(k), self._stream())
         return out
 
-    def _own_rows(self, n: int, k: int) -> int:
-        """Up to how many rows of x the weight-streaming kernel takes a bfloat16 product of this
-        weight; beyond, the library product runs.  Measured on the layer shapes of an 8B model:
-        up to 16 rows the kernel is as fast or faster for every weight; up to 64 rows only for
-        small weights, where the library's kernels leave the GPU half empty."""
-        if 2 * n * k <= self.small_weight_bytes:
-            return self.skinny_max_rows
-        return self.own_matmul_rows
+    def _own_kernel(self, m: int, n: int, k: int) -> Optional[str]:
+        """Which of the engine's weight-streaming kernels takes a bfloat16 product of m rows with a
+        weight [n, k]: "skinny", "medium", or None for the library product.  Measured on the layer
+        shapes of an 8B model: up to 16 rows the skinny kernel is as fast or faster for every
+        weight; up to 128 rows the medium kernel wins for weights of few rows (the library has no
+        split of k and leaves most of the GPU idle there: o and down projections take twice as
+        long), and loses for wide ones (gate/up); small wide weights stay with the skinny kernel
+        up to 64 rows."""
+        if m <= 0:
+            return None
+        if m <= self.own_matmul_rows:
+            return "skinny"
+        if m <= self.medium_max_rows and n <= self.medium_max_weight_rows:
+            return "medium"
+        if m <= self.skinny_max_rows and 2 * n * k <= self.small_weight_bytes:
+            return "skinny"
+        return None
 
     @staticmethod
     def _skinny_takes(x, xs, weight, ws, k) -> bool:
@@ -324,13 +341,36 @@ class HipKernels:
             return SplitSum(self, scratch, used.value, m, n, bias)
         return out
 
+    def _linear_medium(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k, defer=False):
+        """The weight-streaming kernel for up to 128 rows (see _linear_skinny for the arguments)."""
+        rt = self.medium_row_tiles
+        tiles = (n + 15) // 16
+        wgs = (tiles + 4 * rt - 1) // (4 * rt)
+        splits = max(1, min((self.medium_target_workgroups + wgs - 1) // wgs, k // 256))
+        if swiglu and bias is None and 2 * wgs >= self.medium_target_workgroups:
+            splits = 1
+        if defer and splits == 1:
+            defer = False
+            out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+            os_ = n
+        direct = splits == 1 and bias is None
+        scratch = None if direct else torch.empty(splits * m * n, dtype=torch.float32, device=x.device)
+        used = ctypes.c_int(0)
+        library.call("gemm_skinny", "bf16", "nva_linear_medium", _p(x), c_i64(xs), _p(weight), c_i64(ws),
+                     None if defer else _p(bias), _p(out), c_i64(os_), c_i32(1 if out_float32 else 0),
+                     c_i32(1 if swiglu else 0), _p(scratch), c_i32(splits), c_i32(rt), c_i32(1 if defer else 0), c_i64(m),
+                     c_i64(n), c_i64(k), ctypes.byref(used), self._stream())
+        if defer:
+            return SplitSum(self, scratch, used.value, m, n, bias)
+        return out
+
     def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         """silu(x @ Wg.T) * (x @ Wu.T) with weight = [Wg; Wu]."""
         x = _t(x)
         m, k, xs = _rows2d(x, "linear input")
         n, wk, ws = _rows2d(weight, "linear weight")
         if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
-                0 < m <= self._own_rows(n, k) and self._skinny_takes(x, xs, weight, ws, k):
+                self._own_kernel(m, n, k) == "skinny" and self._skinny_takes(x, xs, weight, ws, k):
             out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
             self._linear_skinny(x, xs, weight, ws, None, out, n // 2, False, True, m, n, k)
             return out

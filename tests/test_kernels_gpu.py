@@ -139,7 +139,8 @@ def test_linear_bfloat16(hip, ref, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (8, 6144, 4096), (64, 320, 12288), (17, 1000, 264), (33, 24, 8),
                                    (5, 130, 72), (48, 40000, 1288), (20, 40004, 2304), (64, 4096, 4096),
-                                   (2, 1000, 1288), (4, 40004, 2304), (3, 130, 72), (4, 4096, 12288)])
+                                   (2, 1000, 1288), (4, 40004, 2304), (3, 130, 72), (4, 4096, 12288),
+                                   (100, 1000, 264), (128, 4096, 4096), (120, 130, 72), (90, 4100, 1288), (40, 8192, 512)])
 def test_linear_bfloat16_few_rows_streams_the_weights(hip, ref, m, n, k):
     """The decode-step product (few rows, k split over workgroups) against a double product."""
     x, w = _rand((m, k), torch.bfloat16, 21), _rand((n, k), torch.bfloat16, 22, 0.05)
@@ -161,6 +162,28 @@ def test_linear_silu_mul(hip, ref, m, inner, k):
     _close(hip[torch.bfloat16].linear_silu_mul(x, w), ref.linear_silu_mul(x, w), torch.bfloat16)
     xf, wf = x.float(), w.float()
     _close(hip[torch.float32].linear_silu_mul(xf, wf), ref.linear_silu_mul(xf, wf), torch.float32)
+
+
+@pytest.mark.parametrize("row_tiles", [1, 2])
+@pytest.mark.parametrize("m,n,k,splits", [(128, 512, 1024, 1), (70, 200, 264, 2), (17, 4096, 4096, 8), (97, 72, 8, 1)])
+def test_the_kernel_for_medium_row_counts_in_every_form(hip, m, n, k, splits, row_tiles):
+    """Unsplit and split over k, one and two blocks of weight rows per wave, plain and gated."""
+    kern = hip[torch.bfloat16]
+    x, w = _rand((m, k), torch.bfloat16, 41), _rand((n, k), torch.bfloat16, 42, 0.05)
+    want = x.double() @ w.double().T
+    old = kern.medium_row_tiles, kern.medium_target_workgroups
+    kern.medium_row_tiles = row_tiles
+    kern.medium_target_workgroups = splits * ((n + 15) // 16 + 4 * row_tiles - 1) // (4 * row_tiles)
+    try:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+        kern._linear_medium(x, k, w, k, None, out, n, False, False, m, n, k)
+        _close(out, want.float().to(torch.bfloat16), torch.bfloat16)
+        gated = torch.empty((m, n // 2), dtype=torch.bfloat16, device=DEV)
+        kern._linear_medium(x, k, w, k, None, gated, n // 2, False, True, m, n, k)
+        y = want.float().to(torch.bfloat16).float()
+        _close(gated, (torch.nn.functional.silu(y[:, :n // 2]) * y[:, n // 2:]).to(torch.bfloat16), torch.bfloat16)
+    finally:
+        kern.medium_row_tiles, kern.medium_target_workgroups = old
 
 
 def test_split_products_are_consumed_by_norm_and_qk_kernels(hip, ref):
@@ -199,6 +222,13 @@ def test_split_products_are_consumed_by_norm_and_qk_kernels(hip, ref):
     q2 = k.qk_norm_rope_store(full, hq, hkv, D, qn, kn, 1e-6, table, positions, slots, *caches[1])
     assert torch.equal(q1, q2) and torch.equal(caches[0][0], caches[1][0]) and torch.equal(caches[0][1], caches[1][1])
     assert float(caches[0][1].abs().sum()) > 0
+    # the same for a product of more rows, which the kernel for medium row counts leaves
+    x = _rand((40, kk), torch.bfloat16, 38)
+    y = k.linear(x, w, deferred=True)
+    assert isinstance(y, SplitSum) and y.splits > 1
+    done = k.linear(x, w)
+    assert torch.equal(y.tensor(), done)
+    assert torch.equal(k.rms_norm(y, nw, 1e-6), k.rms_norm(done, nw, 1e-6))
 
 
 # ------------------------------------------------------------------------------ rotation and cache write
