@@ -1,6 +1,7 @@
-// y[M, N] = x[M, K] W[N, K]^T for few rows (M <= 64, bfloat16): the linear layers of a decode
-// step (nanovllm/layers/linear.py:51,73,153; embed_head.py:61), where every weight is read once
-// and the time is the time to stream W from HBM.
+// y[M, N] = x[M, K] W[N, K]^T for few rows (bfloat16): the linear layers of a decode step
+// (nanovllm/layers/linear.py:51,73,153; embed_head.py:61), where every weight is read once and the
+// time is the time to stream W from HBM.  Two kernels: linear_skinny_kernel for up to 64 rows of x
+// (described first), linear_medium_kernel for up to 128.
 //
 // One wave owns 16 output columns (16 rows of W) over a range of k.  W rows are the A operand of
 // a 16x16x32 MFMA, 16 rows of x its 16 columns (rows >= M idle); with more than 16 rows of x the

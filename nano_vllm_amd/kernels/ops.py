@@ -245,8 +245,8 @@ class HipKernels:
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                out_float32: bool = False, out: Optional[torch.Tensor] = None, deferred: bool = False):
         """y = x @ weight.T (+ bias), weight [out, in].  float32 inputs run the engine's own
-        float kernel; bfloat16 inputs with many rows run the library product, with few rows the
-        weight-streaming kernel.  deferred: the caller hands the result to a norm or to the q/k
+        float kernel; bfloat16 inputs with many rows run the library product (also for a float
+        result of more than 16 rows), with few rows the weight-streaming kernels.  deferred: the caller hands the result to a norm or to the q/k
         preparation only, so a product split over k may come back as a SplitSum."""
         x = _t(x)
         m, k, xs = _rows2d(x, "linear input")
@@ -258,6 +258,19 @@ class HipKernels:
         out_dtype = torch.float32 if out_float32 else x.dtype
         if x.dtype == torch.bfloat16 and self._skinny_takes(x, xs, weight, ws, k):
             own = self._own_kernel(m, n, k)
+            if out_float32 and m > self.own_matmul_rows:
+                # logits of many places: the library product with a float result reads the weight
+                # once, where the streaming kernel would read it once per 64 rows
+                y = torch.mm(x, weight.t(), out_dtype=torch.float32)
+                if bias is not None:
+                    y += bias.float()
+                if out is not None:
+                    om, on, _ = _rows2d(out, "linear output")
+                    if (om, on) != (m, n) or out.dtype != out_dtype:
+                        raise KernelError("linear: output does not match")
+                    out.copy_(y)
+                    return out
+                return y
             run = self._linear_medium if own == "medium" else self._linear_skinny
             if deferred and own and not out_float32 and out is None and self.fuse_split_sums:
                 return run(x, xs, weight, ws, bias, None, 0, False, False, m, n, k, defer=True)
