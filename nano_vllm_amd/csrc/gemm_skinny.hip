@@ -204,8 +204,9 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
 // direct and the layout of the results: as above.
 #define MD_KC 128
 #define MD_XS (MD_KC + 8)
+#define MD_WAVES 4
 template <int MB, int RT>
-__global__ void __launch_bounds__(4 * NVA_WAVE) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ void __launch_bounds__(MD_WAVES * NVA_WAVE) __attribute__((amdgpu_waves_per_eu(2)))
 linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf16* __restrict__ w, int64_t w_stride,
                      float* __restrict__ partial, void* __restrict__ y, int64_t y_stride, int y_is_f32, int direct,
                      int M, int N, int K, int k_per_split) {
@@ -220,7 +221,7 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     const bool gated = direct == 2;
     const int inner = N / 2;
     const int per_tile = gated ? 8 : 16;
-    const int tile0 = (blockIdx.x * 4 + wave) * RT;
+    const int tile0 = (blockIdx.x * MD_WAVES + wave) * RT;
     const int k_last = K - 8;
 
     const __bf16* wrow[RT];
@@ -238,24 +239,25 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) acc[rt][b] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    // staging: thread t moves the 16-byte piece t % 16 of rows t / 16 + 16 * j
+    // staging: thread t moves the 16-byte piece t % 16 of rows t / 16 + SR * j
+    constexpr int SR = MD_WAVES * NVA_WAVE / 16, SJ = 16 * MB / SR;
     const int s_row = threadIdx.x / 16, s_piece = threadIdx.x % 16;
-    bf16x8 xr[MB];
+    bf16x8 xr[SJ];
     // (every load of the loop is unconditional, from an address moved into the operand where it
     // would lie outside, and what must be zero is made zero when it is written to LDS: a branch
     // around a load makes the compiler wait for all loads in flight at every turn)
     auto fetch_x = [&](int k0) {
 #pragma unroll
-        for (int j = 0; j < MB; ++j)
-            xr[j] = *reinterpret_cast<const bf16x8*>(x + (int64_t)min(s_row + 16 * j, M - 1) * x_stride +
+        for (int j = 0; j < SJ; ++j)
+            xr[j] = *reinterpret_cast<const bf16x8*>(x + (int64_t)min(s_row + SR * j, M - 1) * x_stride +
                                                      min(k0 + 8 * s_piece, k_last));
     };
     auto store_x = [&](int buf, int k0) {
         const bool k_ok = k0 + 8 * s_piece < k_end;
 #pragma unroll
-        for (int j = 0; j < MB; ++j)
-            *reinterpret_cast<bf16x8*>(&x_s[(buf * ROWS + s_row + 16 * j) * MD_XS + 8 * s_piece]) =
-                k_ok && s_row + 16 * j < M ? xr[j] : zero8();
+        for (int j = 0; j < SJ; ++j)
+            *reinterpret_cast<bf16x8*>(&x_s[(buf * ROWS + s_row + SR * j) * MD_XS + 8 * s_piece]) =
+                k_ok && s_row + SR * j < M ? xr[j] : zero8();
     };
     // W of two chunks is in registers or on its way at any time (16 KiB per wave with RT = 2): with
     // so few waves per CU, less in flight does not cover the memory's latency
@@ -285,18 +287,33 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
         const int k_next = k_of(c + 1), k_ahead = k_of(c + 2);
         fetch_x(k_next);
         const __bf16* xb = x_s + H * ROWS * MD_XS;
+        // The fragments of x come from LDS in groups of GS, one group ahead of the products that use
+        // them: with one or two waves per SIMD nothing else covers the latency of LDS.
+        constexpr int GS = MB % 4 == 0 ? 4 : 2, GROUPS = 4 * MB / GS;          // groups of a chunk: (piece p, blocks b)
+        bf16x8 frag[2][GS];
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
+        for (int i = 0; i < GS; ++i) frag[0][i] = *reinterpret_cast<const bf16x8*>(xb + xoff[i]);
 #pragma unroll
-            for (int b = 0; b < MB; ++b) {
-                const bf16x8 frag = *reinterpret_cast<const bf16x8*>(xb + xoff[b] + 32 * p);
+        for (int gi = 0; gi < GROUPS; ++gi) {
+            constexpr int PER_P = MB / GS;
+            const int p = gi / PER_P, b0 = gi % PER_P * GS;
+            if (gi + 1 < GROUPS) {
+                const int pn = (gi + 1) / PER_P, bn = (gi + 1) % PER_P * GS;
+#pragma unroll
+                for (int i = 0; i < GS; ++i)
+                    frag[(gi + 1) & 1][i] = *reinterpret_cast<const bf16x8*>(xb + xoff[bn + i] + 32 * pn);
+            }
+            __builtin_amdgcn_sched_barrier(0);                        // keep the reads ahead of the products
+#pragma unroll
+            for (int i = 0; i < GS; ++i)
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
-                    acc[rt][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[H][rt][p], frag, acc[rt][b], 0, 0, 0);
-            }
+                    acc[rt][b0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[H][rt][p], frag[gi & 1][i], acc[rt][b0 + i], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (gi % PER_P == PER_P - 1)
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt)      // past the last chunk all lanes read one piece of the first row
-                a[H][rt][p] = *reinterpret_cast<const bf16x8*>((c + 2 < chunks ? wrow[rt] : w + 8 * g) + min(k_ahead + 32 * p, k_last - 8 * g));
+                for (int rt = 0; rt < RT; ++rt)  // past the last chunk all lanes read one piece of the first row
+                    a[H][rt][p] = *reinterpret_cast<const bf16x8*>((c + 2 < chunks ? wrow[rt] : w + 8 * g) + min(k_ahead + 32 * p, k_last - 8 * g));
         }
         store_x(H ^ 1, k_next);                                      // after the last chunk: written, never read
         __syncthreads();
@@ -469,10 +486,10 @@ NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const voi
     const size_t lds = (size_t)2 * (16 * mb + 1) * MD_XS * sizeof(__bf16);
 #define LAUNCH(MB, RT)                                                                                                 \
     do {                                                                                                               \
-        dim3 grid((unsigned)((tiles + 4 * RT - 1) / (4 * RT)), (unsigned)real_splits);                                 \
-        hipLaunchKernelGGL((linear_medium_kernel<MB, RT>), grid, dim3(4 * NVA_WAVE), lds, stream, (const __bf16*)x,    \
-                           x_stride, (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32, direct, (int)M,       \
-                           (int)N, (int)K, kps);                                                                       \
+        dim3 grid((unsigned)((tiles + MD_WAVES * RT - 1) / (MD_WAVES * RT)), (unsigned)real_splits);                   \
+        hipLaunchKernelGGL((linear_medium_kernel<MB, RT>), grid, dim3(MD_WAVES * NVA_WAVE), lds, stream,               \
+                           (const __bf16*)x, x_stride, (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32,     \
+                           direct, (int)M, (int)N, (int)K, kps);                                                       \
     } while (0)
 #define LAUNCH_RT(MB)                                                                                                  \
     do {                                                                                                               \
