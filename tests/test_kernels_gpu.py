@@ -415,6 +415,22 @@ def test_attention_over_long_contexts_matrix_core_kernels_against_the_general_ke
     """Tens of thousands of keys: the bfloat16 matrix-core kernels (decode with splits, prefill
     with its block table in LDS) against the general kernel, which the short cases above pin to
     the plain implementation.  The cache is filled directly; the tables are a random permutation."""
+    _matrix_core_against_general(hip, page, lens, q_lens, window)
+
+
+@pytest.mark.parametrize("page,count,longest,window,seed", [
+    (64, 1100, 300, None, 1),       # more single tokens than one launch of the decode kernel takes
+    (16, 300, 700, 37, 2),          # many requests of very different lengths behind a window
+    (256, 200, 3000, None, 3),      # a wave's share of the keys spans several requests, and a request several waves
+    (8, 40, 90, None, 4),           # requests shorter than a chunk of keys
+])
+def test_decode_attention_shares_the_keys_of_many_requests_out_evenly(hip, page, count, longest, window, seed):
+    rng = random.Random(seed)
+    lens = [rng.randint(1, longest) for _ in range(count)]
+    _matrix_core_against_general(hip, page, lens, [1] * count, window)
+
+
+def _matrix_core_against_general(hip, page, lens, q_lens, window):
     hq, hkv, D = 8, 2, 128
     k = hip[torch.bfloat16]
     S = len(lens)
