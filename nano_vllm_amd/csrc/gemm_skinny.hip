@@ -242,50 +242,49 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     // staging: thread t moves the 16-byte piece t % 16 of rows t / 16 + SR * j
     constexpr int SR = MD_WAVES * NVA_WAVE / 16, SJ = 16 * MB / SR;
     const int s_row = threadIdx.x / 16, s_piece = threadIdx.x % 16;
-    bf16x8 xr[SJ];
+    bf16x8 xr[2][SJ];                                                 // x of the next two chunks, on its way
     // (every load of the loop is unconditional, from an address moved into the operand where it
     // would lie outside, and what must be zero is made zero when it is written to LDS: a branch
     // around a load makes the compiler wait for all loads in flight at every turn)
-    auto fetch_x = [&](int k0) {
+    auto fetch_x = [&](int k0, bf16x8* xr) {
 #pragma unroll
         for (int j = 0; j < SJ; ++j)
             xr[j] = *reinterpret_cast<const bf16x8*>(x + (int64_t)min(s_row + SR * j, M - 1) * x_stride +
                                                      min(k0 + 8 * s_piece, k_last));
     };
-    auto store_x = [&](int buf, int k0) {
+    auto store_x = [&](int buf, int k0, const bf16x8* xr) {
         const bool k_ok = k0 + 8 * s_piece < k_end;
 #pragma unroll
         for (int j = 0; j < SJ; ++j)
             *reinterpret_cast<bf16x8*>(&x_s[(buf * ROWS + s_row + SR * j) * MD_XS + 8 * s_piece]) =
                 k_ok && s_row + SR * j < M ? xr[j] : zero8();
     };
-    // W of two chunks is in registers or on its way at any time (16 KiB per wave with RT = 2): with
-    // so few waves per CU, less in flight does not cover the memory's latency
     // Workgroups walk their chunks in rotated order, each from another start: at one k the rows of
     // x (a power of two apart, as a rule) lie in few channels of the L2, and workgroups that all
     // fetch the same chunk at the same time queue up there.
     const int rot = (blockIdx.x * 5 + blockIdx.y) % chunks;
     // (past the last chunk: K, from where every load is moved back to the rows' last pieces)
     auto k_of = [&](int c) { return c < chunks ? k_begin + (c + rot) % chunks * MD_KC : K; };
-    bf16x8 a[2][RT][4];
-    fetch_x(k_of(0));
+    // x is asked for two chunks ahead (a chunk's products take less time than a load from the L2),
+    // every piece of W one chunk ahead, as soon as its products are issued
+    bf16x8 a[RT][4];
+    fetch_x(k_of(0), xr[0]);
+    fetch_x(k_of(1), xr[1]);
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-            for (int c = 0; c < 4; ++c)
-                a[h][rt][c] = *reinterpret_cast<const bf16x8*>(wrow[rt] + min(k_of(h) + 32 * c, k_last - 8 * g));
+        for (int c = 0; c < 4; ++c)
+            a[rt][c] = *reinterpret_cast<const bf16x8*>(wrow[rt] + min(k_of(0) + 32 * c, k_last - 8 * g));
     if (threadIdx.x < 2 * (MD_XS / 8)) {                              // the row beyond the staged ones, in both halves
         const int buf = threadIdx.x / (MD_XS / 8), piece = threadIdx.x % (MD_XS / 8);
         *reinterpret_cast<bf16x8*>(&x_s[(buf * ROWS + ROWS - 1) * MD_XS + 8 * piece]) = zero8();
     }
-    store_x(0, k_of(0));
+    store_x(0, k_of(0), xr[0]);
     __syncthreads();
     auto chunk = [&](int c, auto half) {
-        constexpr int H = decltype(half)::value;                      // the half of x_s and of `a` this chunk uses
+        constexpr int H = decltype(half)::value;                      // the half of x_s this chunk reads
         const int k_next = k_of(c + 1), k_ahead = k_of(c + 2);
-        fetch_x(k_next);
+        fetch_x(k_ahead, xr[H]);                                      // xr[H ^ 1] holds the next chunk's
         const __bf16* xb = x_s + H * ROWS * MD_XS;
         // The fragments of x come from LDS in groups of GS, one group ahead of the products that use
         // them: with one or two waves per SIMD nothing else covers the latency of LDS.
@@ -308,14 +307,14 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
             for (int i = 0; i < GS; ++i)
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)
-                    acc[rt][b0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[H][rt][p], frag[gi & 1][i], acc[rt][b0 + i], 0, 0, 0);
+                    acc[rt][b0 + i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt][p], frag[gi & 1][i], acc[rt][b0 + i], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             if (gi % PER_P == PER_P - 1)
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt)  // past the last chunk all lanes read one piece of the first row
-                    a[H][rt][p] = *reinterpret_cast<const bf16x8*>((c + 2 < chunks ? wrow[rt] : w + 8 * g) + min(k_ahead + 32 * p, k_last - 8 * g));
+                    a[rt][p] = *reinterpret_cast<const bf16x8*>((c + 1 < chunks ? wrow[rt] : w + 8 * g) + min(k_next + 32 * p, k_last - 8 * g));
         }
-        store_x(H ^ 1, k_next);                                      // after the last chunk: written, never read
+        store_x(H ^ 1, k_next, xr[H ^ 1]);                                    // after the last chunk: written, never read
         __syncthreads();
     };
     for (int c = 0; c < chunks; c += 2) {

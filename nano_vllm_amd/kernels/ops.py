@@ -359,9 +359,9 @@ class HipKernels:
         rt = self.medium_row_tiles
         tiles = (n + 15) // 16
         wgs = (tiles + 4 * rt - 1) // (4 * rt)
-        splits = max(1, min((self.medium_target_workgroups + wgs - 1) // wgs, k // 256))
-        if swiglu and bias is None and 2 * wgs >= self.medium_target_workgroups:
-            splits = 1
+        # as many ranges of k as give at most one workgroup per CU: a second, partly filled round of
+        # workgroups costs more than CUs left idle
+        splits = max(1, min(self.medium_target_workgroups // wgs, k // 256))
         if defer and splits == 1:
             defer = False
             out = torch.empty((m, n), dtype=x.dtype, device=x.device)
