@@ -1,7 +1,7 @@
 // y[M, N] = x[M, K] W[N, K]^T for few rows (bfloat16): the linear layers of a decode step
 // (nanovllm/layers/linear.py:51,73,153; embed_head.py:61), where every weight is read once and the
 // time is the time to stream W from HBM.  Two kernels: linear_skinny_kernel for up to 64 rows of x
-// (described first), linear_medium_kernel for up to 128.
+// (described first), linear_medium_kernel for up to 256.
 //
 // One wave owns 16 output columns (16 rows of W) over a range of k.  W rows are the A operand of
 // a 16x16x32 MFMA, 16 rows of x its 16 columns (rows >= M idle); with more than 16 rows of x the
@@ -195,7 +195,7 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     }
 }
 
-// The same product for more rows of x (up to 128), where the slice of x no longer fits LDS for a
+// The same product for more rows of x (up to 256), where the slice of x no longer fits LDS for a
 // long range of k and the reads of x from LDS weigh as much as the products.  A workgroup of four
 // waves takes 16 * RT rows of W per wave and walks its k range in chunks of 128: the chunk of x
 // lies in LDS twice (the next one is fetched into registers during the products and written to
@@ -205,8 +205,9 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
 #define MD_KC 128
 #define MD_XS (MD_KC + 8)
 #define MD_WAVES 4
+#define MD_MAX_ROWS 256
 template <int MB, int RT>
-__global__ void __launch_bounds__(MD_WAVES * NVA_WAVE) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ void __launch_bounds__(MD_WAVES * NVA_WAVE) __attribute__((amdgpu_waves_per_eu(MB > 8 ? 1 : 2)))
 linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf16* __restrict__ w, int64_t w_stride,
                      float* __restrict__ partial, void* __restrict__ y, int64_t y_stride, int y_is_f32, int direct,
                      int M, int N, int K, int k_per_split) {
@@ -242,7 +243,8 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     // staging: thread t moves the 16-byte piece t % 16 of rows t / 16 + SR * j
     constexpr int SR = MD_WAVES * NVA_WAVE / 16, SJ = 16 * MB / SR;
     const int s_row = threadIdx.x / 16, s_piece = threadIdx.x % 16;
-    bf16x8 xr[2][SJ];                                                 // x of the next two chunks, on its way
+    constexpr int XD = MB > 8 ? 1 : 2;                                // chunks that x is asked for ahead (registers allowing)
+    bf16x8 xr[XD][SJ];                                                // x of the next chunks, on its way
     // (every load of the loop is unconditional, from an address moved into the operand where it
     // would lie outside, and what must be zero is made zero when it is written to LDS: a branch
     // around a load makes the compiler wait for all loads in flight at every turn)
@@ -269,7 +271,6 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     // every piece of W one chunk ahead, as soon as its products are issued
     bf16x8 a[RT][4];
     fetch_x(k_of(0), xr[0]);
-    fetch_x(k_of(1), xr[1]);
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
@@ -280,11 +281,13 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
         *reinterpret_cast<bf16x8*>(&x_s[(buf * ROWS + ROWS - 1) * MD_XS + 8 * piece]) = zero8();
     }
     store_x(0, k_of(0), xr[0]);
+    if (XD == 2) fetch_x(k_of(1), xr[XD - 1]);
     __syncthreads();
     auto chunk = [&](int c, auto half) {
         constexpr int H = decltype(half)::value;                      // the half of x_s this chunk reads
         const int k_next = k_of(c + 1), k_ahead = k_of(c + 2);
-        fetch_x(k_ahead, xr[H]);                                      // xr[H ^ 1] holds the next chunk's
+        if (XD == 2) fetch_x(k_ahead, xr[H % XD]);                    // xr[H ^ 1] holds the next chunk's
+        else fetch_x(k_next, xr[0]);
         const __bf16* xb = x_s + H * ROWS * MD_XS;
         // The fragments of x come from LDS in groups of GS, one group ahead of the products that use
         // them: with one or two waves per SIMD nothing else covers the latency of LDS.
@@ -314,7 +317,7 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
                 for (int rt = 0; rt < RT; ++rt)  // past the last chunk all lanes read one piece of the first row
                     a[rt][p] = *reinterpret_cast<const bf16x8*>((c + 1 < chunks ? wrow[rt] : w + 8 * g) + min(k_next + 32 * p, k_last - 8 * g));
         }
-        store_x(H ^ 1, k_next, xr[H ^ 1]);                                    // after the last chunk: written, never read
+        store_x(H ^ 1, k_next, xr[(H ^ 1) % XD]);                                    // after the last chunk: written, never read
         __syncthreads();
     };
     for (int c = 0; c < chunks; c += 2) {
@@ -460,16 +463,17 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     return nva_check_launch("linear_skinny_finish");
 }
 
-// The kernel for up to 128 rows of x.  row_tiles: 1 or 2 blocks of 16 rows of W per wave.  The other
+// The kernel for up to 256 rows of x.  row_tiles: 1 or 2 blocks of 16 rows of W per wave (always 1
+// beyond 128 rows).  The other
 // arguments as for nva_linear_skinny; k per range is rounded up to a multiple of 128.
 NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
                                       const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
                                       float* scratch, int splits, int row_tiles, int defer_finish, int64_t M,
                                       int64_t N, int64_t K, int* splits_used, hipStream_t stream) {
     if (M == 0 || N == 0) return 0;
-    if (M < 0 || M > 128 || K % 8 || K <= 0 || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
-        nva_fail("linear_medium: needs 1..128 rows, K %% 8 == 0 and 16-byte aligned rows (M=%lld K=%lld)", (long long)M,
-                 (long long)K);
+    if (M < 0 || M > MD_MAX_ROWS || K % 8 || K <= 0 || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
+        nva_fail("linear_medium: needs 1..%d rows, K %% 8 == 0 and 16-byte aligned rows (M=%lld K=%lld)", MD_MAX_ROWS,
+                 (long long)M, (long long)K);
         return 1;
     }
     if (N > 0x7fffffff || K > 0x7fffffff || splits < 1 || splits > 65535) return nva_fail("linear_medium: bad sizes");
@@ -495,11 +499,15 @@ NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const voi
         if (row_tiles == 1) LAUNCH(MB, 1);                                                                             \
         else LAUNCH(MB, 2);                                                                                            \
     } while (0)
-    switch (mb) {
+    switch (mb) {                      // more than 128 rows: one block of weight rows per wave (registers)
         case 2: LAUNCH_RT(2); break;
         case 4: LAUNCH_RT(4); break;
         case 6: LAUNCH_RT(6); break;
-        default: LAUNCH_RT(8); break;
+        case 8: LAUNCH_RT(8); break;
+        case 10: LAUNCH(10, 1); break;
+        case 12: LAUNCH(12, 1); break;
+        case 14: LAUNCH(14, 1); break;
+        default: LAUNCH(16, 1); break;
     }
 #undef LAUNCH_RT
 #undef LAUNCH

@@ -121,7 +121,7 @@ class HipKernels:
         self.own_matmul_rows = 16           # bfloat16 products with more rows go to the library ...
         self.skinny_max_rows = 64           # ... unless the weight is small (see _own_rows); the kernel's limit
         self.small_weight_bytes = 64 << 20
-        self.medium_max_rows = 128          # rows of x the kernel for medium row counts takes
+        self.medium_max_rows = 224          # rows of x the kernel for medium row counts is used for (it takes 256)
         self.medium_max_weight_rows = 8192  # and the widest weight it is used for
         self.medium_row_tiles = 2           # blocks of 16 weight rows per wave in the kernel for up to 128 rows
         self.medium_target_workgroups = 256 # its k range is split until about this many workgroups run (one per CU)
@@ -308,10 +308,10 @@ class HipKernels:
         """Which of the engine's weight-streaming kernels takes a bfloat16 product of m rows with a
         weight [n, k]: "skinny", "medium", or None for the library product.  Measured on the layer
         shapes of an 8B model: up to 16 rows the skinny kernel is as fast or faster for every
-        weight; up to 128 rows the medium kernel wins for weights of few rows (the library has no
+        weight; up to 224 rows the medium kernel wins for weights of few rows (the library has no
         split of k and leaves most of the GPU idle there: o and down projections take twice as
-        long), and loses for wide ones (gate/up); small wide weights stay with the skinny kernel
-        up to 64 rows."""
+        long; at 256 rows the library's tiles fit and it draws level), and loses for wide ones
+        (gate/up); small wide weights stay with the skinny kernel up to 64 rows."""
         if m <= 0:
             return None
         if m <= self.own_matmul_rows:
@@ -355,8 +355,8 @@ class HipKernels:
         return out
 
     def _linear_medium(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k, defer=False):
-        """The weight-streaming kernel for up to 128 rows (see _linear_skinny for the arguments)."""
-        rt = self.medium_row_tiles
+        """The weight-streaming kernel for up to 256 rows (see _linear_skinny for the arguments)."""
+        rt = self.medium_row_tiles if m <= 128 else 1      # more rows: the kernel's registers hold one block
         tiles = (n + 15) // 16
         wgs = (tiles + 4 * rt - 1) // (4 * rt)
         # as many ranges of k as give at most one workgroup per CU: a second, partly filled round of

@@ -140,7 +140,8 @@ def test_linear_bfloat16(hip, ref, m, n, k):
 @pytest.mark.parametrize("m,n,k", [(1, 4096, 4096), (8, 6144, 4096), (64, 320, 12288), (17, 1000, 264), (33, 24, 8),
                                    (5, 130, 72), (48, 40000, 1288), (20, 40004, 2304), (64, 4096, 4096),
                                    (2, 1000, 1288), (4, 40004, 2304), (3, 130, 72), (4, 4096, 12288),
-                                   (100, 1000, 264), (128, 4096, 4096), (120, 130, 72), (90, 4100, 1288), (40, 8192, 512)])
+                                   (100, 1000, 264), (128, 4096, 4096), (120, 130, 72), (90, 4100, 1288), (40, 8192, 512),
+                                   (129, 1000, 264), (200, 4096, 4096), (224, 130, 1288), (161, 72, 8)])
 def test_linear_bfloat16_few_rows_streams_the_weights(hip, ref, m, n, k):
     """The decode-step product (few rows, k split over workgroups) against a double product."""
     x, w = _rand((m, k), torch.bfloat16, 21), _rand((n, k), torch.bfloat16, 22, 0.05)
@@ -165,7 +166,8 @@ def test_linear_silu_mul(hip, ref, m, inner, k):
 
 
 @pytest.mark.parametrize("row_tiles", [1, 2])
-@pytest.mark.parametrize("m,n,k,splits", [(128, 512, 1024, 1), (70, 200, 264, 2), (17, 4096, 4096, 8), (97, 72, 8, 1)])
+@pytest.mark.parametrize("m,n,k,splits", [(128, 512, 1024, 1), (70, 200, 264, 2), (17, 4096, 4096, 8), (97, 72, 8, 1),
+                                          (256, 512, 1024, 2), (150, 200, 264, 1), (241, 136, 4096, 4)])
 def test_the_kernel_for_medium_row_counts_in_every_form(hip, m, n, k, splits, row_tiles):
     """Unsplit and split over k, one and two blocks of weight rows per wave, plain and gated."""
     kern = hip[torch.bfloat16]
