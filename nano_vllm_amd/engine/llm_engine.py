@@ -15,7 +15,6 @@ from typing import Dict, List, Optional, Sequence as Seq, Tuple, Union
 import torch
 
 from ..config.engine_config import EngineConfig
-from ..config.model_config import read_config_json
 from ..sampling.params import SamplingParams
 from ..sampling.sampler import Sampler
 from .batch import StepEntry

@@ -20,7 +20,7 @@ from ..kernels import HipKernels
 from ..parts.model import Model, torch_dtype
 from ..weights.loader import load_weights
 from ..weights.random_weights import fill_random_
-from .batch import StepBatch, StepEntry, build_batch
+from .batch import StepEntry, build_batch
 
 
 class ModelRunner:

@@ -16,7 +16,7 @@ Interface of a mixer:
 """
 from __future__ import annotations
 
-from typing import Dict, Mapping, Optional
+from typing import Dict, Mapping
 
 from .base import BuildContext, ParamDecl, Part, Source
 from .registry import register_part

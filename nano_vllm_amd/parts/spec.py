@@ -8,7 +8,7 @@ a part names the model it is in.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, Mapping, Optional, Tuple
+from typing import Any, Mapping, Optional, Tuple
 
 
 @dataclass(frozen=True)
