@@ -42,6 +42,7 @@ class LLMEngine:
                                   enable_prefix_caching=cfg.enable_prefix_caching)
         if not cfg.enforce_eager and self.model.device.type == "cuda":
             self.runner.enable_decode_graphs(min(cfg.max_num_seqs, 512), cfg.max_model_len)
+            self.runner.capture_decode_graphs()          # at start-up, as the reference does (model_runner.py:222)
         eos = [cfg.eos] if cfg.eos >= 0 else list(spec.eos_token_ids) or self._eos_from_generation_config()
         self.tokenizer = None
         self.scheduler = Scheduler(self.runner.cache, cfg.max_num_seqs, cfg.max_num_batched_tokens,

@@ -13,6 +13,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from ..cache.manager import CacheManager, plan_groups
+from ..cache.pages import OutOfPages
 from ..cache import storage
 from ..config.model_config import read_config_json
 from ..config.registry import architecture_of
@@ -40,6 +41,7 @@ class ModelRunner:
         self.layer_caches = storage.allocate(self.needs, self.groups, self.state_runs, counts, page_size,
                                              max_requests, model.dtype, self.device)
         self._graphs = {}
+        self._graph_pool = None
         self._graph_max_batch = 0
         self._graph_max_len = 0
 
@@ -80,6 +82,35 @@ class ModelRunner:
         self._graph_max_len = max_len
         self._graph_table_width = (max_len + self.page_size - 1) // self.page_size
 
+    def capture_decode_graphs(self) -> int:
+        """Captures every batch size now, the largest first (so that the smaller ones find their
+        memory in the shared pool), with stand-in requests of one token each; what cannot be
+        captured for want of pages or request slots is left for its first occurrence.  Returns the
+        number of sizes captured.  (nanovllm/engine/model_runner.py:222-257 does this at start-up.)"""
+        if not self._graph_max_batch or self.device.type != "cuda":
+            return 0
+        sizes = sorted({self.graph_batch_size(n) for n in range(1, self._graph_max_batch + 1)}, reverse=True)
+        done = 0
+        for b in sizes:
+            if b in self._graphs or b > self._graph_max_batch or any(pool.num_free < b for pool in self.cache.pools) \
+                    or (self.cache.slots.num_slots and self.cache.slots.num_free < b):
+                continue
+            names = [("captured decode step", i) for i in range(b)]
+            held = []
+            try:
+                for name in names:
+                    self.cache.admit(name)
+                    held.append(name)
+                    self.cache.reserve(name, 1)
+                self._step_graph([StepEntry(name, [0], 0, [0]) for name in names])
+                done += 1
+            except OutOfPages:
+                pass
+            finally:
+                for name in held:
+                    self.cache.release(name)
+        return done
+
     def _graph_takes(self, entries) -> bool:
         if len(entries) > self._graph_max_batch or self.device.type != "cuda":
             return False
@@ -119,7 +150,9 @@ class ModelRunner:
             torch.cuda.current_stream(self.device).wait_stream(side)
             torch.cuda.synchronize(self.device)
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            if self._graph_pool is None:                  # one memory pool for all sizes: they run one at a time
+                self._graph_pool = torch.cuda.graph_pool_handle()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
                 logits = self.model.logits(self.model.forward(batch, self.layer_caches), batch.logits_rows)
             g = (graph, static, logits, batch)
             self._graphs[size_b] = g

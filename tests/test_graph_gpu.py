@@ -107,3 +107,39 @@ def test_a_burst_of_decode_steps_gives_the_tokens_of_single_steps(dtype):
         runs.append(toks)
     assert runs[0] == runs[1]
     assert all(len(runs[1][rid]) == len(reqs[rid]) + 1 + 19 for rid in reqs)
+
+
+def test_graphs_captured_at_start_give_the_eager_steps():
+    """Every batch size captured up front with stand-in requests (largest first, one memory pool):
+    no page or slot stays held, and a later step of real requests replays what an eager step gives."""
+    c = H.CONFIGS["b"]
+    folder = H.model_folder("b", "float32")
+    eager = H.make_runner(folder, "float32", c["page"], 40)
+    graphed = H.make_runner(folder, "float32", c["page"], 40)
+    graphed.enable_decode_graphs(max_batch=8, max_len=c["cfg"].max_position_embeddings)
+    assert graphed.capture_decode_graphs() == 4 and sorted(graphed._graphs) == [1, 2, 4, 8]
+    graphed.cache.check()
+    assert graphed.cache.pools[0].num_free == 40
+    assert graphed.capture_decode_graphs() == 0                        # nothing left to capture
+    V = c["cfg"].vocab_size
+    reqs = {f"r{i}": H.random_tokens(V, 30, 50 + i) for i in range(3)}
+    for r in (eager, graphed):
+        for rid, toks in reqs.items():
+            r.cache.admit(rid)
+            r.cache.reserve(rid, 25)
+            r.step([StepEntry(rid, toks[:25], 0, [])])
+    for pos in range(25, 30):
+        outs = []
+        for r in (eager, graphed):
+            entries = []
+            for rid in reqs:
+                r.cache.reserve(rid, pos + 1)
+                entries.append(StepEntry(rid, [reqs[rid][pos]], pos, [0]))
+            outs.append(r.step(entries).clone())
+            torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]), f"replay at position {pos} differs from the eager step"
+    # too few pages for the largest sizes: they are left for their first occurrence
+    small = H.make_runner(folder, "float32", c["page"], 5)
+    small.enable_decode_graphs(max_batch=8, max_len=c["cfg"].max_position_embeddings)
+    assert small.capture_decode_graphs() == 3 and sorted(small._graphs) == [1, 2, 4]
+    graphed.kernels.check_faults()
