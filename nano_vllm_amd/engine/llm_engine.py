@@ -72,6 +72,11 @@ class LLMEngine:
                                                   if len(d.shape) == 2 and d.shape[0] < model.spec.vocab_size])
         activations = cfg.max_num_batched_tokens * (4 * widest + 8 * model.spec.hidden_size) * itemsize
         activations += cfg.max_num_seqs * model.spec.vocab_size * 4 * 2
+        if not cfg.enforce_eager:
+            # every captured decode step keeps its own logits: one row per request of its batch size
+            top = min(cfg.max_num_seqs, 512)
+            rows = sum({ModelRunner.graph_batch_size(n) for n in range(1, top + 1)})
+            activations += rows * model.spec.vocab_size * 4
         budget = int(total * cfg.gpu_memory_utilization) - used - activations
         pages = budget // max(per_page, 1)
         if pages <= 0:
