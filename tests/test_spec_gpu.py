@@ -100,7 +100,7 @@ def test_layer_sizes_of_the_8b_shape(tmp_path, dtype):
     pcfg, w = plain.read_folder(folder)
     want = plain.logits(w, pcfg, toks, None if dtype == "float32" else "bfloat16")
     tol = 2e-5 if dtype == "float32" else 2e-2
-    for portions in ([n], [n - 32] + [1] * 32, [250, 2, 7, 41]):
+    for portions in ([n], [n - 32] + [1] * 32, [250, 2, 7, 41], [100, 200]):       # 41, 100, 200 rows: the kernel for medium row counts
         got = H.run_portions(r, "x", toks, portions)
         assert H.rel_err(got, want) < tol, portions
     r.kernels.check_faults()
