@@ -464,7 +464,7 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
 }
 
 // The kernel for up to 256 rows of x.  row_tiles: 1 or 2 blocks of 16 rows of W per wave (always 1
-// beyond 128 rows).  The other
+// beyond 224 rows).  The other
 // arguments as for nva_linear_skinny; k per range is rounded up to a multiple of 128.
 NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
                                       const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
@@ -499,14 +499,14 @@ NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const voi
         if (row_tiles == 1) LAUNCH(MB, 1);                                                                             \
         else LAUNCH(MB, 2);                                                                                            \
     } while (0)
-    switch (mb) {                      // more than 128 rows: one block of weight rows per wave (registers)
+    switch (mb) {                      // more than 224 rows: one block of weight rows per wave (registers)
         case 2: LAUNCH_RT(2); break;
         case 4: LAUNCH_RT(4); break;
         case 6: LAUNCH_RT(6); break;
         case 8: LAUNCH_RT(8); break;
-        case 10: LAUNCH(10, 1); break;
-        case 12: LAUNCH(12, 1); break;
-        case 14: LAUNCH(14, 1); break;
+        case 10: LAUNCH_RT(10); break;
+        case 12: LAUNCH_RT(12); break;
+        case 14: LAUNCH_RT(14); break;
         default: LAUNCH(16, 1); break;
     }
 #undef LAUNCH_RT

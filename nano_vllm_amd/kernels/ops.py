@@ -356,7 +356,7 @@ class HipKernels:
 
     def _linear_medium(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k, defer=False):
         """The weight-streaming kernel for up to 256 rows (see _linear_skinny for the arguments)."""
-        rt = self.medium_row_tiles if m <= 128 else 1      # more rows: the kernel's registers hold one block
+        rt = self.medium_row_tiles if m <= 224 else 1      # more rows: the kernel's registers hold one block
         tiles = (n + 15) // 16
         wgs = (tiles + 4 * rt - 1) // (4 * rt)
         # as many ranges of k as give at most one workgroup per CU: a second, partly filled round of
