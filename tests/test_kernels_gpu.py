@@ -157,7 +157,8 @@ def test_linear_bfloat16_few_rows_streams_the_weights(hip, ref, m, n, k):
 
 
 @pytest.mark.parametrize("m,inner,k", [(1, 12288, 4096), (8, 200, 96), (64, 160, 256), (100, 64, 128), (5, 8196, 264),
-                                       (40, 9004, 1288), (16, 12288, 4096), (2, 8196, 264), (4, 9004, 1288), (3, 200, 96)])
+                                       (40, 9004, 1288), (16, 12288, 4096), (2, 8196, 264), (4, 9004, 1288), (3, 200, 96),
+                                       (24, 12288, 4096), (32, 8196, 264), (17, 200, 96)])
 def test_linear_silu_mul(hip, ref, m, inner, k):
     x, w = _rand((m, k), torch.bfloat16, 24), _rand((2 * inner, k), torch.bfloat16, 25, 0.1)
     _close(hip[torch.bfloat16].linear_silu_mul(x, w), ref.linear_silu_mul(x, w), torch.bfloat16)
