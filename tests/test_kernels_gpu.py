@@ -407,6 +407,56 @@ def test_paged_attention(hip, ref, dtype, hq, hkv, D, page, lens, q_lens, window
             hip[dtype].mfma_attention = True
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_attention_of_drawn_shapes(hip, ref, seed):
+    """Head counts, groups, head sizes, page sizes, windows and lengths drawn at random (single tokens
+    first, as the engine orders a step): the bfloat16 kernels against the plain whole-sequence attention."""
+    rng = random.Random(1000 + seed)
+    hkv = rng.choice([1, 2, 3, 5])
+    G = rng.choice([1, 2, 3, 4, 7, 8, 16])
+    D = rng.choice([32, 64, 96, 128, 160, 256])
+    page = rng.choice([8, 16, 24, 64])
+    window = rng.choice([None, None, 5, 33, 100])
+    decodes = rng.randint(1, 12)
+    lens = [rng.randint(1, 300) for _ in range(decodes)]
+    q_lens = [1] * decodes
+    for _ in range(rng.randint(0, 2)):
+        n = rng.randint(2, 200)
+        lens.append(n + rng.choice([0, 0, rng.randint(1, 150)]))
+        q_lens.append(n)
+    dtype = torch.bfloat16
+    q, kc, vc, batch, parts = _paged_case(dtype, hkv * G, hkv, D, page, lens, q_lens, seed=200 + seed)
+    scale = D ** -0.5
+    got = hip[dtype].paged_attention(q, hkv * G, hkv, D, kc, vc, batch, 0, scale, window)
+    want = _plain_attention(*parts, lens, q_lens, scale, window).to(DEV)
+    _close(got, want.to(dtype), dtype, f"hkv {hkv} group {G} head_dim {D} page {page} window {window} lens {lens} q {q_lens}")
+    hip[dtype].check_faults()
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_products_of_drawn_shapes(hip, ref, seed):
+    """Rows, widths and depths drawn at random over the ranges of the weight-streaming kernels (k a
+    multiple of 8, anything else free), plain, with a bias, with a float result, left as partial sums."""
+    from nano_vllm_amd.kernels.ops import SplitSum
+    rng = random.Random(2000 + seed)
+    m = rng.choice([rng.randint(1, 16), rng.randint(17, 128), rng.randint(129, 256)])
+    n = rng.choice([rng.randint(1, 300), rng.randint(1000, 9000)])
+    k = 8 * rng.choice([rng.randint(1, 40), rng.randint(100, 700)])
+    kern = hip[torch.bfloat16]
+    x, w = _rand((m, k), torch.bfloat16, 3000 + seed), _rand((n, k), torch.bfloat16, 3100 + seed, 0.05)
+    b = _rand((n,), torch.bfloat16, 3200 + seed)
+    want = x.double() @ w.double().T
+    what = f"m {m} n {n} k {k}"
+    _close(kern.linear(x, w), want.float().to(torch.bfloat16), torch.bfloat16, what)
+    _close(kern.linear(x, w, b), (want + b.double()).float().to(torch.bfloat16), torch.bfloat16, what + " with a bias")
+    bound = (x.double().abs() @ w.double().abs().T) * (math.sqrt(k) * 2.0 ** -23) + 1e-30
+    assert bool(((kern.linear(x, w, out_float32=True).double() - want).abs() <= bound).all()), what + " float result"
+    y = kern.linear(x, w, b, deferred=True)
+    if isinstance(y, SplitSum):
+        assert torch.equal(y.tensor(), kern.linear(x, w, b)), what + " deferred"
+    kern.check_faults()
+
+
 @pytest.mark.parametrize("page,lens,q_lens,window", [
     (256, [40000, 12345, 257, 4096], [1, 1, 1, 1], None),           # long decoding: 157 pages in a table
     (16, [30000, 5000], [1, 1], None),                              # the same over small pages: splits capped by pages
