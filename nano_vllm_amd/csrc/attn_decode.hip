@@ -439,6 +439,54 @@ attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restri
     }
 }
 
+// The same merge with one wave per (token, head) and four pairs per workgroup: for steps of many
+// tokens, where there are pairs enough to fill the GPU and a token has few segments.
+__global__ void __launch_bounds__(MERGE_WAVES * NVA_WAVE)
+attn_decode_merge_wave_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                              const int32_t* __restrict__ plan, __bf16* __restrict__ out, int64_t out_stride,
+                              int tokens, int num_q_heads, int head_dim) {
+    const int lane = threadIdx.x % NVA_WAVE;
+    const int64_t pair = (int64_t)blockIdx.x * MERGE_WAVES + threadIdx.x / NVA_WAVE;
+    if (pair >= (int64_t)tokens * num_q_heads) return;
+    const int64_t t = pair / num_q_heads;
+    const int head = (int)(pair % num_q_heads);
+    const int s_lo = plan[2 + t], s_hi = plan[2 + t + 1] - 1;
+    if (s_hi <= s_lo) return;
+    auto slot_of = [&](int s) { return (int64_t)s * num_q_heads + head; };
+    float m = -INFINITY;
+    for (int s = s_lo + lane; s <= s_hi; s += NVA_WAVE) m = fmaxf(m, part_ml[slot_of(s) * 2]);
+    m = wave_max(m);
+    float l = 0.f;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = s_lo; s0 <= s_hi; s0 += 4) {
+        float wj[4], v[4][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int s = min(s0 + j, s_hi);                              // a segment past the end: read again, weight 0
+            const float ms = part_ml[slot_of(s) * 2];
+            wj[j] = (s0 + j > s_hi || ms == -INFINITY) ? 0.f : __expf(ms - m);
+            l += part_ml[slot_of(s) * 2 + 1] * wj[j];
+            const float* po = part_o + slot_of(s) * head_dim;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = lane + i * NVA_WAVE;
+                v[j][i] = d < head_dim ? po[d] : 0.f;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += v[j][i] * wj[j];
+    }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    __bf16* orow = out + t * out_stride + (int64_t)head * head_dim;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int d = lane + i * NVA_WAVE;
+        if (d < head_dim) orow[d] = (__bf16)(acc[i] * inv);
+    }
+}
+
 // What the decode attention of `tokens` single tokens needs when no request holds more than `longest`
 // keys: the bound of the segments of all tokens together, the number of persistent waves (a multiple
 // of the kv heads), and the size of the plan (int32).  Partial results: max_segments * num_q_heads *
@@ -521,6 +569,13 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
 #undef LAUNCH
     int rc = nva_check_launch("attn_decode");
     if (rc) return rc;
+    const int64_t pairs = tokens * num_q_heads;
+    if (pairs >= 2 * DEC_RESIDENT_WAVES) {            // pairs enough for a wave each
+        hipLaunchKernelGGL(attn_decode_merge_wave_kernel, dim3((unsigned)((pairs + MERGE_WAVES - 1) / MERGE_WAVES)),
+                           dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, plan, (__bf16*)out, out_stride,
+                           (int)tokens, num_q_heads, head_dim);
+        return nva_check_launch("attn_decode_merge");
+    }
     dim3 mgrid((unsigned)tokens, (unsigned)num_q_heads);
     hipLaunchKernelGGL(attn_decode_merge_kernel, mgrid, dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, plan,
                        (__bf16*)out, out_stride, num_q_heads, head_dim);
