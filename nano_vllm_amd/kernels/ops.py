@@ -335,7 +335,9 @@ class HipKernels:
         target = self.skinny_target_waves if m <= 16 else self.skinny_target_waves // 2
         # few rows of x: staging them costs little, and four waves that share rows of the weight and
         # split k between them inside the workgroup leave fewer partial sums to add
-        kw = self.skinny_waves_per_tile or (4 if m <= 4 else 1)
+        # (a gate/up product of up to 16 rows: two waves share the rows, which makes waves enough to
+        # leave k unsplit, so that the gating happens in the product kernel and no partial sums are written)
+        kw = self.skinny_waves_per_tile or (4 if m <= 4 else 2 if swiglu and bias is None and m <= 16 else 1)
         splits = max(1, min((target + tiles * kw - 1) // (tiles * kw), k // 256))
         if swiglu and bias is None and 2 * tiles * kw >= target:
             splits = 1          # wide enough without a split of k: the gating happens in the product kernel
