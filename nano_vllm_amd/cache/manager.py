@@ -131,6 +131,17 @@ class CacheManager:
         give = self._passed_pages(request, first_query)
         return all(pool.num_free + g >= n for pool, n, g in zip(self.pools, need, give))
 
+    def can_reserve_all(self, wanted: Sequence[Tuple[Hashable, int, Optional[int]]]) -> bool:
+        """Whether reserve() would succeed for every (request, new_len, first_query) of `wanted`,
+        one after the other: all of them, or none, is what a caller needs who must not keep
+        pages for some requests when others find none."""
+        need = [0] * len(self.pools)
+        for request, new_len, first_query in wanted:
+            for g, (n, give) in enumerate(zip(self.pages_needed(request, new_len, first_query),
+                                              self._passed_pages(request, first_query))):
+                need[g] += n - give
+        return all(pool.num_free >= n for pool, n in zip(self.pools, need))
+
     def _passed_pages(self, request, first_query) -> List[int]:
         rc = self.requests[request]
         first_query = rc.num_tokens if first_query is None else first_query

@@ -16,8 +16,8 @@
 // A token whose keys lie in several quotas gets an unnormalised partial result (max, sum, O) from
 // each; a second kernel merges them.  A token inside one quota is written by the first kernel itself.
 //
-// Requires head_dim % 32 == 0 (32..256), G <= 16, page_size % 8 == 0; the launcher refuses
-// anything else and the caller falls back to the general kernel.
+// Requires head_dim % 32 == 0 (32..256), G <= 16, page_size % 8 == 0.  The launcher refuses anything
+// else with an error; the host wrapper knows these limits and runs the general kernel instead.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -524,8 +524,8 @@ NVA_EXPORT int nva_attn_decode_plan_bf16(const int32_t* positions, const int32_t
     return nva_check_launch("attn_decode_plan");
 }
 
-// Returns 1 (and leaves a message) for shapes this kernel does not take; the caller then uses the
-// general kernel.  plan: made by nva_attn_decode_plan for these tokens, kv heads, page size and
+// Refuses (non-zero code and a message) shapes this kernel does not take: the host wrapper checks
+// the same limits first and runs the general kernel for them.  plan: made by nva_attn_decode_plan for these tokens, kv heads, page size and
 // window; max_segments and waves from nva_attn_decode_plan_size.
 NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride, float* scratch,
                                     const int32_t* plan, const void* k_cache, const void* v_cache,

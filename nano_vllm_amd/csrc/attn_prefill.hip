@@ -16,8 +16,9 @@
 // sixteen scores a lane holds per tile are keys 8h..8h+7 and 16+8h..16+8h+7: two operands of the
 // second product as they are.
 //
-// Requires head_dim % 32 == 0 (32..256) and page_size % 8 == 0; the launcher refuses anything else
-// and the caller falls back to the general kernel.
+// Requires head_dim % 32 == 0 (32..256), page_size % 8 == 0 and block tables of at most 4096 pages
+// (the table row is staged in LDS).  The launcher refuses anything else with an error; the host
+// wrapper knows these limits and runs the general kernel instead.
 #include "common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -320,7 +321,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
 
 // tiles: int32 [num_tiles][2] = (request, row tile of 32 queries) for every tile of the step's
 // portions, ordered from the most visible keys to the fewest (the caller builds it once per step).
-// Returns 1 (and leaves a message) for shapes this kernel does not take.
+// Refuses (non-zero code and a message) shapes this kernel does not take.
 NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out, int64_t out_stride,
                                      const void* k_cache, const void* v_cache, const int32_t* block_tables,
                                      int table_stride, const int32_t* cu_seqlens_q, const int32_t* kv_lens,

@@ -407,7 +407,7 @@ linear_skinny_finish_kernel(const float* __restrict__ partial, int splits, const
 // waves_per_tile: 1, 2 or 4 waves of a workgroup share 16 rows of W and split the k range between
 // them (pays for very few rows of x).  splits: how many ranges k is cut into (>= 1); scratch must hold splits * M * N floats when
 // splits > 1 or a bias, swiglu or defer_finish is asked for.  splits_used receives the number of
-// ranges really used (k per range is rounded up to a multiple of 256).  Returns 1 for shapes this kernel does not take.
+// ranges really used (k per range is rounded up to a multiple of 256).  Refuses (non-zero code and a message) shapes this kernel does not take.
 NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
                                       const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
                                       float* scratch, int splits, int waves_per_tile, int defer_finish, int64_t M,

@@ -300,7 +300,8 @@ static int launch_qk(elem_t* qkv, int64_t row_stride, PartialInput part, elem_t*
 
 // qkv rows hold [q heads | k heads | v heads] of head_dim each.  q_weight / k_weight may be null
 // (no norm), table may be null (no rotation), the caches may be null (nothing is stored).
-// Positions are checked on the host against the rows of the table.
+// The kernels read table + positions[t] * head_dim unchecked: the host wrapper takes the largest
+// position of the step and refuses one that is not a row of the table.
 NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store)(void* qkv, int64_t row_stride, int64_t tokens, int num_q_heads,
                                                 int num_kv_heads, int head_dim, const void* q_weight,
                                                 const void* k_weight, int w_is_f32, float eps, const float* table,

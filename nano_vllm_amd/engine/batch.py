@@ -57,7 +57,7 @@ class StepBatch:
 
 def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size: int, device,
                 table_width: Optional[int] = None, static: Optional[torch.Tensor] = None,
-                pad_to: Optional[int] = None) -> StepBatch:
+                pad_to: Optional[int] = None, max_position: Optional[int] = None) -> StepBatch:
     """Orders the entries (single tokens first), checks them against the cache manager's
     block tables and uploads everything in one copy.
 
@@ -67,7 +67,9 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
     width the layout is the same for every step, which is what a captured graph replays on.
     pad_to (decoded tokens only) fills the batch up to that many requests with copies of the
     first entry that write nothing into the cache (slot -1): they read what the first request
-    reads, and their logits, which follow the real ones, are dropped by the caller."""
+    reads, and their logits, which follow the real ones, are dropped by the caller.
+    max_position: the positions the model knows (rows of its position tables); an entry that
+    reaches beyond is refused here, since the kernels read those tables unchecked."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
@@ -98,6 +100,9 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
         if e.start < 0 or e.start + n > rc.num_tokens:
             raise ValueError(f"request {e.request!r}: positions {e.start}..{e.start + n - 1} are not reserved "
                              f"in the cache ({rc.num_tokens} are)")
+        if max_position is not None and e.start + n > max_position:
+            raise ValueError(f"request {e.request!r}: position {e.start + n - 1} is beyond the model's "
+                             f"{max_position} positions (max_position_embeddings)")
         cu.append(cu[-1] + n)
         kv_lens.append(e.start + n)
         starts.append(e.start)

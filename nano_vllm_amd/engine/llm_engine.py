@@ -177,18 +177,20 @@ class LLMEngine:
         runner = self.runner
         if not (getattr(runner, "_graph_max_batch", 0) and runner._graph_takes(entries)):
             return 1
+        if len(runner.groups) > getattr(self.model.kernels, "max_burst_groups", 0):
+            return 1            # the kernel that advances a step's metadata on the device takes so many groups
         for s in seqs:
             if s.num_cached_tokens + 1 != s.num_tokens:
                 return 1
             want = min(want, s.max_tokens - s.num_completion_tokens, self.config.max_model_len - s.num_tokens)
         if want <= 1:
             return 1
-        from ..cache import OutOfPages
-        try:
-            for s in seqs:
-                self.runner.cache.reserve(s.seq_id, s.num_tokens + want - 1, first_query=s.num_tokens - 1)
-        except OutOfPages:
+        # all requests or none: a request must not keep pages for steps that will not run
+        wanted = [(s.seq_id, s.num_tokens + want - 1, s.num_tokens - 1) for s in seqs]
+        if not runner.cache.can_reserve_all(wanted):
             return 1
+        for request, new_len, first_query in wanted:
+            runner.cache.reserve(request, new_len, first_query=first_query)
         return want
 
     def generate(self, prompts: Seq[Union[str, List[int]]],

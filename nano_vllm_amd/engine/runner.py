@@ -63,7 +63,8 @@ class ModelRunner:
         step of the same batch size.)"""
         if self._graph_max_batch and self._graph_takes(entries):
             return self._step_graph(entries)
-        batch = build_batch(entries, self.cache, self.page_size, self.model.spec.vocab_size, self.device)
+        batch = build_batch(entries, self.cache, self.page_size, self.model.spec.vocab_size, self.device,
+                            max_position=self.model.spec.max_position)
         hidden = self.model.forward(batch, self.layer_caches)
         if batch.logits_rows is None:
             return None
@@ -78,6 +79,8 @@ class ModelRunner:
         which captures every size at start-up."""
         if self.state_runs:
             return          # a mixer with host-side state handling cannot be replayed blindly
+        if max_len > self.model.spec.max_position:
+            raise ValueError(f"decode graphs for {max_len} tokens: the model knows {self.model.spec.max_position} positions")
         self._graph_max_batch = max_batch
         self._graph_max_len = max_len
         self._graph_table_width = (max_len + self.page_size - 1) // self.page_size
@@ -140,7 +143,8 @@ class ModelRunner:
             size = 3 * b + (b + 1) + 3 * b + b + num_groups * (b + b * self._graph_table_width)
             static = torch.zeros(size, dtype=torch.int32, device=self.device)
             batch = build_batch(entries, self.cache, self.page_size, vocab, self.device,
-                                table_width=self._graph_table_width, static=static, pad_to=size_b)
+                                table_width=self._graph_table_width, static=static, pad_to=size_b,
+                                max_position=self.model.spec.max_position)
             batch.max_kv_len = self._graph_max_len        # launch shapes must cover every later step
             side = torch.cuda.Stream(self.device)
             side.wait_stream(torch.cuda.current_stream(self.device))
@@ -158,7 +162,8 @@ class ModelRunner:
             self._graphs[size_b] = g
         graph, static, logits, _ = g
         build_batch(entries, self.cache, self.page_size, vocab, self.device,
-                    table_width=self._graph_table_width, static=static, pad_to=size_b)
+                    table_width=self._graph_table_width, static=static, pad_to=size_b,
+                    max_position=self.model.spec.max_position)
         graph.replay()
         return logits[:n]
 

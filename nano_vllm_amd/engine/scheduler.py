@@ -13,7 +13,9 @@ When pages run out:
   * a running request that needs a page for its next token takes it from the request that
     was admitted last: that one is preempted - its pages are given back, it returns to the
     front of the waiting queue and is computed again from its tokens, prompt and generated
-    (scheduler.py:60-65,75-79);
+    (scheduler.py:60-65,75-79); under "mixed" the request admitted last may still be at the
+    head of the waiting queue with a part of its prompt in the cache, and is then the first
+    to give its pages back;
   * a request that is alone and still cannot grow is finished with reason "cache_full"
     (the reference asserts, scheduler.py:71); a prompt that can never fit the pool is
     refused when it is added.
@@ -102,7 +104,11 @@ class Scheduler:
         while self.running and len(batch) < self.max_num_seqs:
             seq = self.running.popleft()
             while not self.cache.can_reserve(seq.seq_id, seq.num_tokens, first_query=seq.num_tokens - 1):
-                if self.running:
+                if self.waiting and self.waiting[0].admitted:
+                    # policy "mixed": the request admitted last is still being cut into portions and
+                    # holds pages at the head of the waiting queue; it is the newest, so it goes first
+                    self._preempt_waiting_head()
+                elif self.running:
                     self.preempt(self.running.pop())
                 elif batch:
                     self.preempt(seq)
@@ -130,13 +136,21 @@ class Scheduler:
 
     def preempt(self, seq: Sequence) -> None:
         """scheduler.py:75-79."""
+        self._take_pages_away(seq)
+        self.waiting.appendleft(seq)
+
+    def _preempt_waiting_head(self) -> None:
+        """The same for a request that holds pages but has not left the waiting queue yet (its
+        prompt is not all in the cache): it keeps its place at the head."""
+        self._take_pages_away(self.waiting[0])
+
+    def _take_pages_away(self, seq: Sequence) -> None:
         self.num_preemptions += 1
         seq.status = SequenceStatus.WAITING
         self.cache.release(seq.seq_id)
         seq.admitted = False
         seq.num_cached_tokens = 0
         seq.num_scheduled_tokens = 0
-        self.waiting.appendleft(seq)
 
     # ------------------------------------------------------------------ after the step
     def postprocess(self, seqs: Seq[Sequence], token_ids: Seq[int]) -> None:

@@ -85,7 +85,20 @@ def _t(x):
     return x.tensor() if isinstance(x, SplitSum) else x
 
 
+def check_positions_fit(table: torch.Tensor, head_dim: int, max_position: Optional[int]) -> None:
+    """The rotary kernels read row positions[t] of the table without a check on the device: a
+    step whose positions are not all rows of the table is refused here."""
+    if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != head_dim or not table.is_contiguous():
+        raise KernelError(f"rotary table must be float32 [positions, {head_dim}]: partial rotation is not built")
+    if max_position is None:
+        raise KernelError("rotation by a table needs max_position, the bound of the step's positions")
+    if max_position > table.shape[0]:
+        raise KernelError(f"a position of {max_position - 1} has no row in the rotary table of {table.shape[0]} "
+                          f"positions (max_position_embeddings)")
+
+
 PREFILL_ROWS = 32       # query rows of one workgroup of the prefill attention kernel
+PREFILL_MAX_TABLE = 4096    # pages of a block-table row the prefill attention kernel stages in LDS
 
 
 def prefill_tile_order(q_lens, starts, first_seq: int) -> list:
@@ -105,6 +118,7 @@ class HipKernels:
     """Every device operation of the engine.  Needs a GPU and the compiled libraries."""
 
     name = "hip"
+    max_burst_groups = 4        # cache groups nva_advance_decode takes in one launch
 
     def __init__(self, device="cuda:0", dtype: torch.dtype = torch.bfloat16, quiet: bool = False):
         if not torch.cuda.is_available():
@@ -115,7 +129,8 @@ class HipKernels:
         self.dtype = dtype
         self.suffix = _SUFFIX[dtype]
         library.preload(self.suffix, quiet=quiet)       # compiles what this element type needs
-        # bit 0: a token id outside the vocabulary; bit 1: a visible key without a page
+        # bit 0: a token id outside the vocabulary; bit 1: a visible key without a page;
+        # bit 2: the decode attention's plan outgrew its bound
         self.fault_flag = torch.zeros(1, dtype=torch.int32, device=self.device)
         # Rows up to which the bfloat16 product runs on the engine's own kernels.
         self.own_matmul_rows = 16           # bfloat16 products with more rows go to the library ...
@@ -145,6 +160,10 @@ class HipKernels:
                 what.append("a token id outside the vocabulary reached the embedding")
             if flags & 2:
                 what.append("attention met a visible key whose page is missing from the block table")
+            if flags & 4:
+                what.append("the decode attention's plan needed more segments than it was sized for")
+            if flags & ~7:
+                what.append(f"unknown flags {flags & ~7:#x}")
             raise KernelError("device-side check failed: " + "; ".join(what))
 
     # ------------------------------------------------------------------ rows
@@ -406,9 +425,13 @@ class HipKernels:
                            q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
                            table: Optional[torch.Tensor], positions: Optional[torch.Tensor],
                            slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
-                           v_cache: Optional[torch.Tensor]) -> torch.Tensor:
+                           v_cache: Optional[torch.Tensor], max_position: Optional[int] = None) -> torch.Tensor:
         """Per-head norm of q and k, rotation by the table's rows, q and k written back in
-        place, k and v written into their page slots.  Returns the q view [T, heads*head_dim]."""
+        place, k and v written into their page slots.  Returns the q view [T, heads*head_dim].
+        max_position: every entry of `positions` lies below it (the caller knows the step's
+        largest position on the host); needed with a table, whose rows the kernel reads unchecked."""
+        if table is not None:
+            check_positions_fit(table, head_dim, max_position)
         if isinstance(qkv, SplitSum):
             return self._qk_of_partials(qkv, num_heads, num_kv_heads, head_dim, q_weight, k_weight, eps, table,
                                         positions, slots, k_cache, v_cache)
@@ -425,8 +448,6 @@ class HipKernels:
         if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
             raise KernelError("qk norm: the two weights differ in type")
         if table is not None:
-            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != head_dim or not table.is_contiguous():
-                raise KernelError(f"rotary table must be float32 [positions, {head_dim}]: partial rotation is not built")
             _i32(positions, tokens, "positions")
         page_size = 0
         if k_cache is not None:
@@ -452,8 +473,6 @@ class HipKernels:
         if q_weight is not None and k_weight is not None and q_weight.dtype != k_weight.dtype:
             raise KernelError("qk norm: the two weights differ in type")
         if table is not None:
-            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != head_dim or not table.is_contiguous():
-                raise KernelError(f"rotary table must be float32 [positions, {head_dim}]")
             _i32(positions, tokens, "positions")
         page_size = 0
         if k_cache is not None:
@@ -517,7 +536,7 @@ class HipKernels:
             self._attention_decode(q, qs, out, os_, k_cache, v_cache, tables, batch, start, num_heads, num_kv_heads,
                                    head_dim, page_size, scale, window)
         if start < tokens and q.dtype == torch.bfloat16 and self.mfma_attention and start == batch.num_decode and \
-                self._decode_kernel_takes(1, head_dim, page_size, q, qs, out, os_):
+                self._prefill_kernel_takes(head_dim, page_size, tables.shape[1], q, qs, out, os_):
             # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
             tiles = getattr(batch, "prefill_tiles", None)
             if tiles is None:       # a batch that was not built by the engine: order the tiles here, once
@@ -545,8 +564,15 @@ class HipKernels:
 
     @staticmethod
     def _decode_kernel_takes(group, head_dim, page_size, q, q_stride, out, out_stride) -> bool:
+        """The limits of nva_attn_decode; what it does not take runs the general kernel."""
         return (group <= 16 and head_dim % 32 == 0 and 32 <= head_dim <= 256 and page_size % 8 == 0
                 and q.data_ptr() % 16 == 0 and q_stride % 8 == 0 and out.data_ptr() % 16 == 0 and out_stride % 8 == 0)
+
+    @classmethod
+    def _prefill_kernel_takes(cls, head_dim, page_size, table_width, q, q_stride, out, out_stride) -> bool:
+        """The limits of nva_attn_prefill (head sizes, page size, the block-table row it stages)."""
+        return table_width <= PREFILL_MAX_TABLE and cls._decode_kernel_takes(1, head_dim, page_size, q, q_stride, out,
+                                                                             out_stride)
 
     def _attention_decode(self, q, qs, out, os_, k_cache, v_cache, tables, batch, n, num_heads, num_kv_heads,
                           head_dim, page_size, scale, window):
@@ -610,8 +636,8 @@ class HipKernels:
         _i32(sampled, n_real, "sampled")
         _i32(out_row, n_real, "out_row")
         groups = batch.groups
-        if len(groups) > 4:
-            raise KernelError("advance_decode: at most 4 cache groups")
+        if len(groups) > self.max_burst_groups:
+            raise KernelError(f"advance_decode: at most {self.max_burst_groups} cache groups")
         ptr = ctypes.c_void_p * max(len(groups), 1)
         widths = (ctypes.c_int * max(len(groups), 1))(*[g.block_tables.shape[1] for g in groups])
         for g in groups:

@@ -92,7 +92,7 @@ class Attention(Part):
         kw = w.get("k_norm.weight")
         if pe is None or table is not None:
             q = k.qk_norm_rope_store(qkv, self.heads, kv_heads, self.head_dim, qw, kw, self.eps, table,
-                                     batch.positions, slots, kc, vc)
+                                     batch.positions, slots, kc, vc, max_position=batch.max_kv_len)
         else:
             # an encoding without a table: norm, the part's own encoding, then the store
             q = k.qk_norm_rope_store(qkv, self.heads, kv_heads, self.head_dim, qw, kw, self.eps, None, None,

@@ -216,3 +216,17 @@ def test_state_slots():
     pool.give_back(s)
     with pytest.raises(PageError):
         pool.give_back(s)
+
+
+def test_reserving_for_several_requests_is_all_or_nothing():
+    m = CacheManager([CacheGroup(None, (0,))], 4, 5)
+    for r, n in (("a", 7), ("b", 8)):
+        m.admit(r)
+        m.reserve(r, n)
+    assert m.pools[0].num_free == 1
+    assert m.can_reserve_all([("a", 8, 7), ("b", 8, 7)])             # no new page
+    assert m.can_reserve_all([("a", 12, 7), ("b", 8, 7)])            # one new page: it is there
+    assert not m.can_reserve_all([("a", 12, 7), ("b", 12, 7)])       # two are not, though each alone would find one
+    assert m.can_reserve("a", 12, 7) and m.can_reserve("b", 12, 7)
+    assert m.pools[0].num_free == 1
+    m.check()

@@ -1,0 +1,65 @@
+"""Host-side decisions of the kernel wrappers that need no GPU: which attention kernel takes
+a shape, which product kernel takes a row count, what the fault flags say, and the check of
+positions against the rotary table."""
+import pytest
+import torch
+
+from nano_vllm_amd.kernels.library import KernelError
+from nano_vllm_amd.kernels.ops import HipKernels, PREFILL_MAX_TABLE, check_positions_fit
+
+
+def _qo(rows=4, width=256):
+    q = torch.zeros((rows, width), dtype=torch.bfloat16)
+    return q, width, torch.zeros_like(q), width
+
+
+def test_prefill_kernel_is_not_chosen_for_block_tables_it_cannot_stage():
+    q, qs, out, os_ = _qo()
+    takes = HipKernels._prefill_kernel_takes
+    assert takes(128, 256, 16, q, qs, out, os_)
+    assert takes(128, 8, PREFILL_MAX_TABLE, q, qs, out, os_)
+    # pages of 8 tokens and a context of more than 32768: the general kernel runs instead
+    assert not takes(128, 8, PREFILL_MAX_TABLE + 1, q, qs, out, os_)
+    assert not takes(16, 4, 8, q, qs, out, os_)           # head size 16, pages of 4
+    assert not takes(128, 4, 8, q, qs, out, os_)
+    assert not takes(128, 256, 8, q, 252, out, os_)       # rows that are not 16-byte aligned
+
+
+def test_decode_kernel_limits():
+    q, qs, out, os_ = _qo()
+    takes = HipKernels._decode_kernel_takes
+    assert takes(4, 128, 256, q, qs, out, os_) and takes(16, 32, 8, q, qs, out, os_)
+    assert not takes(17, 128, 256, q, qs, out, os_)       # more than 16 query heads per kv head
+    assert not takes(4, 48, 256, q, qs, out, os_) and not takes(4, 288, 256, q, qs, out, os_)
+    assert not takes(4, 128, 12, q, qs, out, os_)
+
+
+def test_every_fault_flag_has_a_message():
+    k = object.__new__(HipKernels)
+    for flags, text in ((1, "token id"), (2, "page is missing"), (4, "plan needed more segments"), (8, "unknown flags")):
+        k.fault_flag = torch.tensor([flags], dtype=torch.int32)
+        with pytest.raises(KernelError, match=text):
+            k.check_faults()
+        assert int(k.fault_flag) == 0
+    k.check_faults()
+
+
+def test_positions_must_be_rows_of_the_rotary_table():
+    table = torch.zeros((128, 16))
+    check_positions_fit(table, 16, 128)
+    with pytest.raises(KernelError, match="no row in the rotary table of 128"):
+        check_positions_fit(table, 16, 129)
+    with pytest.raises(KernelError, match="needs max_position"):
+        check_positions_fit(table, 16, None)
+    with pytest.raises(KernelError, match="float32"):
+        check_positions_fit(table, 32, 10)
+
+
+def test_row_counts_choose_the_product_kernel():
+    k = object.__new__(HipKernels)
+    # the thresholds are instance attributes set in __init__, which needs a GPU: the defaults, by hand
+    k.own_matmul_rows, k.skinny_max_rows, k.small_weight_bytes = 16, 64, 64 << 20
+    k.medium_max_rows, k.medium_max_weight_rows = 224, 8192
+    assert k._own_kernel(1, 4096, 4096) == "skinny" and k._own_kernel(16, 24576, 4096) == "skinny"
+    assert k._own_kernel(17, 4096, 4096) == "medium" and k._own_kernel(224, 4096, 12288) == "medium"
+    assert k._own_kernel(0, 4096, 4096) is None

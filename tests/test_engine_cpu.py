@@ -157,3 +157,88 @@ def test_temperature_sampling_is_the_plain_draw_and_is_reproducible():
 def test_unknown_option_is_an_error():
     with pytest.raises(TypeError, match="unknown engine options"):
         _llm("a", max_batch=3)
+
+
+def test_step_refuses_a_position_the_model_does_not_know():
+    """The rotary table has max_position_embeddings rows and the kernels read it unchecked:
+    the step function refuses an entry that reaches beyond, whoever calls it."""
+    r = _runner("a", 80)                                   # configuration a knows 128 positions
+    r.cache.admit("x")
+    r.cache.reserve("x", 130)
+    toks = H.random_tokens(256, 130, 3)
+    r.step([StepEntry("x", toks[:128], 0, [127])])         # positions 0..127 are all there
+    with pytest.raises(ValueError, match="beyond the model's 128 positions"):
+        r.step([StepEntry("x", toks[128:129], 128, [0])])
+    r.cache.admit("y")
+    r.cache.reserve("y", 130)
+    with pytest.raises(ValueError, match="beyond the model's 128 positions"):
+        r.step([StepEntry("y", toks, 0, [])])
+    with pytest.raises(ValueError, match="positions"):
+        r.enable_decode_graphs(2, 129)
+
+
+def test_trace_run_refuses_a_trace_longer_than_the_model_knows(tmp_path):
+    """bin/trace_run drives the step function without the scheduler's length limit: a trace
+    that runs past max_position_embeddings ends with an error, not with a read past the table."""
+    import importlib.machinery
+    import importlib.util
+    import io
+    import json
+    import os
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "bin", "trace_run")
+    loader = importlib.machinery.SourceFileLoader("trace_run_program", path)
+    trace_run = importlib.util.module_from_spec(importlib.util.spec_from_loader("trace_run_program", loader))
+    loader.exec_module(trace_run)
+    toks = H.random_tokens(256, 130, 4)
+    lines = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:126], "want": [125]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": toks[126:128], "want": [1]}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": toks[128:130], "want": [0]}], "end": ["a"]}]
+    argv = ["--model", H.model_folder("a"), "--dtype", "float32", "--out", str(tmp_path), "--max-tokens", "256",
+            "--device", "cpu"]
+    with pytest.raises(ValueError, match="beyond the model's 128 positions"):
+        trace_run.main(argv, io.StringIO("\n".join(json.dumps(l) for l in lines) + "\n"), TorchKernels())
+    assert sorted(os.listdir(tmp_path)) == ["0.f32", "1.f32"]          # the steps before it ran
+    want = H.plain_logits(H.model_folder("a"), toks[:128])
+    import numpy as np
+    got = torch.from_numpy(np.fromfile(os.path.join(tmp_path, "1.f32"), dtype="<f4").reshape(1, 256))
+    assert H.rel_err(got, want[127:128]) < TOL
+
+
+def test_a_burst_reserves_for_all_its_requests_or_for_none():
+    """Several decode steps in a row need pages for all of them: when the pool cannot give them
+    to every request of the batch, no request keeps any (single steps follow), and a model
+    with more cache groups than the metadata kernel takes never bursts."""
+    llm = _llm("a", num_kvcache_blocks=6, decode_burst=4, max_num_batched_tokens=32)           # pages of 4 tokens
+    sp = SamplingParams(temperature=0.0, max_tokens=20)
+    for p in _prompts("a", (7, 11)):
+        llm.add_request(p, sp)
+    llm.step()                                                         # both prompts: 2 and 3 pages, 1 free
+    llm.model.kernels.max_burst_groups = 4
+    llm.runner._graph_max_batch = 8                                    # as if decode steps were captured
+    llm.runner._graph_takes = lambda entries: True
+    seqs, is_prefill = llm.scheduler.schedule()                        # decode at positions 7 and 11: no new page
+    assert not is_prefill and len(seqs) == 2
+    entries = [StepEntry(s.seq_id, s.token_ids[-1:], s.num_cached_tokens, [0]) for s in seqs]
+    tables = [list(llm.runner.cache.table(s.seq_id, 0)) for s in seqs]
+    free = llm.runner.cache.pools[0].num_free
+    assert free == 1
+    # steps 2..4 need a third page for the first request (positions 8..10), which is there, and a
+    # fourth for the second (12..14), which is not: the first must not keep the one it could have
+    assert llm._burst_steps(seqs, entries, False) == 1
+    assert llm.runner.cache.pools[0].num_free == free
+    assert [list(llm.runner.cache.table(s.seq_id, 0)) for s in seqs] == tables
+    llm.runner.cache.check()
+    # with pages enough the same call reserves for all steps
+    big = _llm("a", num_kvcache_blocks=16, decode_burst=4)
+    for p in _prompts("a", (7, 8)):
+        big.add_request(p, sp)
+    big.step()
+    big.model.kernels.max_burst_groups = 4
+    big.runner._graph_max_batch = 8
+    big.runner._graph_takes = lambda entries: True
+    seqs, _ = big.scheduler.schedule()
+    entries = [StepEntry(s.seq_id, s.token_ids[-1:], s.num_cached_tokens, [0]) for s in seqs]
+    assert big._burst_steps(seqs, entries, False) == 4
+    assert all(big.runner.cache.requests[s.seq_id].num_tokens == s.num_tokens + 3 for s in seqs)
+    big.model.kernels.max_burst_groups = 0
+    assert big._burst_steps(seqs, entries, False) == 1

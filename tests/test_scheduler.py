@@ -183,3 +183,24 @@ def test_policies_end_with_the_same_tokens(policy):
     if policy == "mixed":
         assert any(len({n for _, _, n in b}) > 1 and any(n == 1 for _, _, n in b) for _, b in log), \
             "no step mixed a prompt portion with decoded tokens"
+
+
+def test_mixed_policy_takes_pages_from_a_prompt_that_is_still_being_cut():
+    """Under "mixed" the request admitted last may hold pages while it is still at the head of
+    the waiting queue (its prompt goes in portions).  A running request that needs a page takes
+    them from it, the newest, instead of ending with "cache_full"; it is computed again later."""
+    def run(policy, pages):
+        s = _sched(pages=pages, page=4, budget=3, policy=policy, prefix=False)
+        a, b = _seq(3, max_tokens=12), _seq(16, 50, max_tokens=3)
+        s.add(a); s.add(b)
+        log = _run(s)
+        return a, b, s, log
+    a, b, s, log = run("mixed", 6)           # a grows to 4 pages while b holds 4 for its 16-token prompt
+    assert s.num_preemptions >= 1
+    assert a.finish_reason == "max_tokens" and a.num_completion_tokens == 12
+    assert b.finish_reason == "max_tokens" and b.num_completion_tokens == 3
+    assert s.cache.pools[0].num_free == 6
+    # b was taken from while part of its prompt was in the cache, and kept its place in the queue
+    assert any(sid == b.seq_id and start > 0 for _, batch in log for sid, start, n in batch)
+    a2, b2, s2, _ = run("prefill_first", 64)
+    assert a.token_ids == a2.token_ids and b.token_ids == b2.token_ids and s2.num_preemptions == 0

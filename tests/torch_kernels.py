@@ -101,7 +101,9 @@ class TorchKernels:
         return torch.cat((ang.cos(), ang.sin()), dim=-1)
 
     def qk_norm_rope_store(self, qkv, num_heads, num_kv_heads, head_dim, q_weight, k_weight, eps, table,
-                           positions, slots, k_cache, v_cache):
+                           positions, slots, k_cache, v_cache, max_position=None):
+        if table is not None:
+            assert max_position is not None and max_position <= table.shape[0], "a position has no row in the table"
         T = qkv.shape[0]
         D = head_dim
         qd, kd = num_heads * D, num_kv_heads * D
