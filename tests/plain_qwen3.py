@@ -1,7 +1,7 @@
 """Plain, slow implementation of the Qwen3 dense decoder: whole sequences, no cache.
 
 Written from the formulas in the reference's text (each function cites file:line
-under /root/reference).  It shares no code with the engine: it reads config.json
+as nanovllm/...).  It shares no code with the engine: it reads config.json
 and model.safetensors itself, keeps q/k/v and gate/up as separate matrices, builds
 a dense causal mask and recomputes everything for every call.
 

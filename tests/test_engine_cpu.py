@@ -20,7 +20,7 @@ def _runner(name, pages):
     return H.make_runner(H.model_folder(name), "float32", c["page"], pages, device="cpu", kernels=TorchKernels())
 
 
-@pytest.mark.parametrize("name", ["a", "b"])
+@pytest.mark.parametrize("name", ["a", "b", "e"])
 def test_every_cutting_gives_the_plain_logits(name):
     c = H.CONFIGS[name]
     n = 70
@@ -242,3 +242,15 @@ def test_a_burst_reserves_for_all_its_requests_or_for_none():
     assert all(big.runner.cache.requests[s.seq_id].num_tokens == s.num_tokens + 3 for s in seqs)
     big.model.kernels.max_burst_groups = 0
     assert big._burst_steps(seqs, entries, False) == 1
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_requests_that_share_prefix_pages_give_the_plain_logits(name):
+    """The drive of tests/test_replay_gpu.py's prefix test on the host side alone: hashed pages are
+    found while in use, found after they were given back, and lost to other requests."""
+    c = H.CONFIGS[name]
+    top = min(c["cfg"].max_position_embeddings - 2, 250)
+    folder = H.model_folder(name)
+    r = H.make_runner(folder, "float32", c["page"], H.prefix_pool_pages(name, top), device="cpu",
+                      kernels=TorchKernels(), prefix_caching=True)
+    H.check_prefix_reuse(r, name, top, lambda toks: H.plain_logits(folder, toks), TOL)

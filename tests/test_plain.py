@@ -91,6 +91,19 @@ def test_rope_is_complex_multiplication_of_half_split_pairs():
     assert torch.allclose(y[: D // 2], z.real, atol=1e-5) and torch.allclose(y[D // 2:], z.imag, atol=1e-5)
 
 
+def test_rope_of_a_vector_worked_by_hand():
+    # head_dim 4, theta 10000: the two frequencies are 1 and 10000^(-2/4) = 0.01 (an exponent of
+    # i/D would give 0.1, one of 2i/(D/2) would give 0.0001); position 3: angles 3 and 0.03.
+    # Pairs (0, 2) and (1, 3) of x = [1, 2, 3, 4]:
+    #   y0 = 1 cos 3 - 3 sin 3      y2 = 3 cos 3 + 1 sin 3      cos 3 = -0.98999250, sin 3 = 0.14112001
+    #   y1 = 2 cos .03 - 4 sin .03  y3 = 4 cos .03 + 2 sin .03  cos .03 = 0.99955003, sin .03 = 0.02999550
+    ang = plain.rope_angles(4, torch.tensor([3]), 10000.0)
+    assert torch.allclose(ang, torch.tensor([[3.0, 0.03]]), rtol=1e-6)
+    y = plain.apply_rope(torch.tensor([[[1.0, 2.0, 3.0, 4.0]]], dtype=torch.float64), ang.double())
+    want = torch.tensor([-1.41335252, 1.87911807, -2.82885748, 4.05819114], dtype=torch.float64)
+    assert torch.allclose(y.view(4), want, atol=1e-6)
+
+
 def test_rope_scores_depend_on_distance_only():
     D = 32
     q, k = torch.randn(1, 1, D, dtype=torch.float64), torch.randn(1, 1, D, dtype=torch.float64)
@@ -186,6 +199,72 @@ def test_zero_output_projections_leave_the_normalised_embedding():
     h0 = w["model.embed_tokens.weight"][torch.tensor(ids)]
     want = plain.rms_norm(h0, w["model.norm.weight"], cfg.rms_norm_eps) @ w["lm_head.weight"].T
     assert torch.allclose(plain.logits(w, cfg, ids), want, atol=1e-12)
+
+
+def _library_model(w, cfg, ids):
+    """The whole decoder put together from library routines only: F.embedding, F.rms_norm,
+    F.linear, torch.polar (the rotation as a complex product), F.scaled_dot_product_attention
+    with is_causal (kv heads repeated for their query heads), F.silu, and the residual written
+    the usual way.  Nothing of tests/plain_qwen3.py is called."""
+    T, D, Hq, Hkv = len(ids), cfg.head_dim, cfg.num_heads, cfg.num_kv_heads
+    x = F.embedding(torch.tensor(ids), w["model.embed_tokens.weight"])
+    pos = torch.arange(T, dtype=torch.float64)
+    freq = torch.tensor([cfg.rope_theta ** (-2.0 * i / D) for i in range(D // 2)], dtype=torch.float64)
+    turn = torch.polar(torch.ones(T, D // 2, dtype=torch.float64), pos[:, None] * freq[None, :])     # [T, D/2]
+
+    def rotate(t):                                               # t [T, heads, D]
+        z = torch.complex(t[..., : D // 2], t[..., D // 2:]) * turn[:, None, :]
+        return torch.cat((z.real, z.imag), dim=-1)
+
+    for i in range(cfg.num_layers):
+        p = f"model.layers.{i}"
+        a = f"{p}.self_attn"
+        y = F.rms_norm(x, (cfg.hidden_size,), w[f"{p}.input_layernorm.weight"], cfg.rms_norm_eps)
+        bias = (lambda n: w[f"{a}.{n}.bias"]) if cfg.attention_bias else (lambda n: None)
+        q = F.linear(y, w[f"{a}.q_proj.weight"], bias("q_proj")).view(T, Hq, D)
+        k = F.linear(y, w[f"{a}.k_proj.weight"], bias("k_proj")).view(T, Hkv, D)
+        v = F.linear(y, w[f"{a}.v_proj.weight"], bias("v_proj")).view(T, Hkv, D)
+        if not cfg.attention_bias:
+            q = F.rms_norm(q, (D,), w[f"{a}.q_norm.weight"], cfg.rms_norm_eps)
+            k = F.rms_norm(k, (D,), w[f"{a}.k_norm.weight"], cfg.rms_norm_eps)
+        q, k = rotate(q), rotate(k)
+        k, v = (t.repeat_interleave(Hq // Hkv, dim=1) for t in (k, v))
+        o = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
+        x = x + F.linear(o.transpose(0, 1).reshape(T, Hq * D), w[f"{a}.o_proj.weight"])
+        y = F.rms_norm(x, (cfg.hidden_size,), w[f"{p}.post_attention_layernorm.weight"], cfg.rms_norm_eps)
+        m = F.silu(F.linear(y, w[f"{p}.mlp.gate_proj.weight"])) * F.linear(y, w[f"{p}.mlp.up_proj.weight"])
+        x = x + F.linear(m, w[f"{p}.mlp.down_proj.weight"])
+    x = F.rms_norm(x, (cfg.hidden_size,), w["model.norm.weight"], cfg.rms_norm_eps)
+    return F.linear(x, w["model.embed_tokens.weight"] if cfg.tie_word_embeddings else w["lm_head.weight"])
+
+
+@pytest.mark.parametrize("kw", [
+    dict(),                                                                        # grouped heads, untied
+    dict(tie_word_embeddings=True, num_heads=6, num_kv_heads=6, head_dim=4, rope_theta=1e6, rms_norm_eps=1e-6),
+    dict(attention_bias=True, num_kv_heads=1, num_layers=3),                       # bias, no q/k norm
+    dict(num_heads=8, num_kv_heads=2, head_dim=16, hidden_size=40, intermediate_size=56, vocab_size=97),
+])
+def test_whole_model_is_the_composition_of_library_routines(kw):
+    """The plain model as a whole against a second one that is made of library routines: a
+    norm in the wrong place, a wrong pairing or direction of the rotation, a wrong head
+    grouping, a missing bias or a q/k norm where there is a bias all fail this.  (The one
+    formula both type is the frequency theta^(-2i/D), which the vector worked by hand pins.)"""
+    cfg = _cfg(**kw)
+    w = _weights(cfg, seed=5)
+    if cfg.attention_bias:
+        g = torch.Generator().manual_seed(9)
+        for i in range(cfg.num_layers):
+            for n, rows in (("q_proj", cfg.num_heads), ("k_proj", cfg.num_kv_heads), ("v_proj", cfg.num_kv_heads)):
+                w[f"model.layers.{i}.self_attn.{n}.bias"] = torch.randn(rows * cfg.head_dim, generator=g).double()
+    ids = torch.randint(0, cfg.vocab_size, (19,), generator=torch.Generator().manual_seed(2)).tolist()
+    got = plain.logits(w, cfg, ids)
+    want = _library_model(w, cfg, ids)
+    # the angles of the plain model are float32, as the reference's table is
+    assert torch.allclose(got, want, atol=1e-5 * float(want.abs().max())), float((got - want).abs().max())
+    if cfg.attention_bias:
+        for i in range(cfg.num_layers):          # the q/k norm weights are there but must not be read
+            w[f"model.layers.{i}.self_attn.q_norm.weight"] *= 3.0
+        assert torch.equal(plain.logits(w, cfg, ids), got)
 
 
 def test_shift_of_all_positions_changes_nothing():

@@ -41,7 +41,7 @@ def _length(name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d", "e"])
 @pytest.mark.parametrize("driving", ["whole", "last32", "portions"])
 def test_one_request(runners, name, dtype, driving):
     n = _length(name)
@@ -57,7 +57,7 @@ def test_one_request(runners, name, dtype, driving):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["b", "c", "d"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d", "e"])
 def test_mixed_requests_on_few_pages(runners, name, dtype):
     c = H.CONFIGS[name]
     top = _length(name)
@@ -71,6 +71,20 @@ def test_mixed_requests_on_few_pages(runners, name, dtype):
         want = H.plain_logits(H.model_folder(name, dtype), toks, ROUNDING[dtype])
         assert H.rel_err(got[rid], want) < TOL[dtype], rid
     assert r.cache.pools[0].num_free == pages
+    r.kernels.check_faults()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_mixed_requests_that_share_prefix_pages(name, dtype):
+    """nanovllm/engine/block_manager.py:58-92,110-120 on the GPU, compared by logits: pages
+    found by their hash while another request holds them, pages found after they were given
+    back, pages that were taken again in between (the prefix is then computed again), on a
+    pool that holds about three requests.  Every computed position against the plain model."""
+    c = H.CONFIGS[name]
+    folder = H.model_folder(name, dtype)
+    r = H.make_runner(folder, dtype, c["page"], H.prefix_pool_pages(name, _length(name)), prefix_caching=True)
+    H.check_prefix_reuse(r, name, _length(name), lambda toks: H.plain_logits(folder, toks, ROUNDING[dtype]), TOL[dtype])
     r.kernels.check_faults()
 
 
