@@ -156,6 +156,30 @@ def test_linear_bfloat16_few_rows_streams_the_weights(hip, ref, m, n, k):
     _close(hip[torch.bfloat16].linear(x, w, b), (want + b.double()).float().to(torch.bfloat16), torch.bfloat16)
 
 
+@pytest.mark.parametrize("m", [1, 8, 17, 64])
+def test_logits_of_a_vocabulary_of_151936(hip, m):
+    """The output head at its real size (151936 x 4096, float result): one row and eight through
+    the weight-streaming kernel, 17 and 64 through the path for many wanted places, each against
+    a double product, and the argmax of every row with it."""
+    n, k = 151936, 4096
+    x = _rand((m, k), torch.bfloat16, 51)
+    gen = torch.Generator(device=DEV).manual_seed(52)
+    w = torch.empty((n, k), dtype=torch.bfloat16, device=DEV).normal_(0, 0.02, generator=gen)
+    got = hip[torch.bfloat16].linear(x, w, out_float32=True)
+    assert got.dtype == torch.float32 and got.shape == (m, n)
+    want = torch.empty((m, n), dtype=torch.float64, device=DEV)
+    bound = torch.empty((m, n), dtype=torch.float64, device=DEV)
+    xd = x.double()
+    for lo in range(0, n, 16384):                      # in slices: the weight in double would not be small
+        wd = w[lo:lo + 16384].double()
+        want[:, lo:lo + 16384] = xd @ wd.T
+        bound[:, lo:lo + 16384] = (xd.abs() @ wd.abs().T) * (math.sqrt(k) * 2.0 ** -23)
+    # every column was written, the last ones too, each within a float sum's rounding
+    assert bool(((got.double() - want).abs() <= bound).all()), float(((got.double() - want).abs() / bound).max())
+    assert torch.equal(got.argmax(-1), want.argmax(-1))
+    hip[torch.bfloat16].check_faults()
+
+
 @pytest.mark.parametrize("m,inner,k", [(1, 12288, 4096), (8, 200, 96), (64, 160, 256), (100, 64, 128), (5, 8196, 264),
                                        (40, 9004, 1288), (16, 12288, 4096), (2, 8196, 264), (4, 9004, 1288), (3, 200, 96),
                                        (24, 12288, 4096), (32, 8196, 264), (17, 200, 96)])
@@ -464,11 +488,12 @@ def test_products_of_drawn_shapes(hip, ref, seed):
     (64, [33000], [1500], 4096),                                    # a window far into a long request
     (256, [16000, 16000, 16000], [1, 1, 300], 1000),
 ])
-def test_attention_over_long_contexts_matrix_core_kernels_against_the_general_kernel(hip, page, lens, q_lens, window):
+def test_attention_over_long_contexts_against_plain_arithmetic(hip, page, lens, q_lens, window):
     """Tens of thousands of keys: the bfloat16 matrix-core kernels (decode with splits, prefill
-    with its block table in LDS) against the general kernel, which the short cases above pin to
-    the plain implementation.  The cache is filled directly; the tables are a random permutation."""
-    _matrix_core_against_general(hip, page, lens, q_lens, window)
+    with its block table in LDS) and the general kernel, each against a float softmax over the
+    keys and values gathered from the pages.  The cache is filled directly; the tables are a
+    random permutation."""
+    _kernels_against_gathered_attention(hip, page, lens, q_lens, window)
 
 
 @pytest.mark.parametrize("page,count,longest,window,seed", [
@@ -480,10 +505,34 @@ def test_attention_over_long_contexts_matrix_core_kernels_against_the_general_ke
 def test_decode_attention_shares_the_keys_of_many_requests_out_evenly(hip, page, count, longest, window, seed):
     rng = random.Random(seed)
     lens = [rng.randint(1, longest) for _ in range(count)]
-    _matrix_core_against_general(hip, page, lens, [1] * count, window)
+    _kernels_against_gathered_attention(hip, page, lens, [1] * count, window)
 
 
-def _matrix_core_against_general(hip, page, lens, q_lens, window):
+def _gathered_attention(q, kc, vc, tables, lens, q_lens, hq, hkv, D, page, scale, window):
+    """Plain float attention of each request's last q_lens tokens over its keys and values, which
+    are gathered from the pages its block table names (K [pages, kv heads, page, D], V in tiles
+    of vt keys [pages, kv heads, page / vt, D, vt]).  Shares nothing with the kernels."""
+    out, row = [], 0
+    G = hq // hkv
+    for s, (n, nq) in enumerate(zip(lens, q_lens)):
+        pages = tables[s, : (n + page - 1) // page].long().to(kc.device)
+        K = kc[pages].float().permute(1, 0, 2, 3).reshape(hkv, -1, D)[:, :n]                    # [hkv, n, D]
+        V = vc[pages].float().permute(1, 0, 2, 4, 3).reshape(hkv, -1, D)[:, :n]                 # tiles -> keys
+        Q = q[row:row + nq].float().view(nq, hkv, G, D).permute(1, 2, 0, 3)                      # [hkv, G, nq, D]
+        scores = torch.einsum("hgqd,hkd->hgqk", Q, K) * scale
+        qpos = torch.arange(n - nq, n, device=kc.device)[:, None]
+        kpos = torch.arange(n, device=kc.device)[None, :]
+        seen = kpos <= qpos
+        if window:
+            seen &= (qpos - kpos) < window
+        scores = scores.masked_fill(~seen, float("-inf"))
+        o = torch.einsum("hgqk,hkd->hgqd", torch.softmax(scores, dim=-1), V)                      # [hkv, G, nq, D]
+        out.append(o.permute(2, 0, 1, 3).reshape(nq, hq * D))
+        row += nq
+    return torch.cat(out)
+
+
+def _kernels_against_gathered_attention(hip, page, lens, q_lens, window):
     hq, hkv, D = 8, 2, 128
     k = hip[torch.bfloat16]
     S = len(lens)
@@ -509,13 +558,15 @@ def _matrix_core_against_general(hip, page, lens, q_lens, window):
         cu_seqlens_q=torch.tensor([0] + list(torch.tensor(q_lens).cumsum(0)), dtype=torch.int32, device=DEV),
         num_decode=next((i for i, n in enumerate(q_lens) if n != 1), len(q_lens)), q_lens=list(q_lens),
         groups=[SimpleNamespace(block_tables=tables.to(DEV), slot_mapping=None)])
+    want = _gathered_attention(q, kc, vc, tables, lens, q_lens, hq, hkv, D, page, D ** -0.5, window)
     got = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, D ** -0.5, window)
+    _close(got, want, torch.bfloat16, "matrix-core kernels against the float softmax over gathered keys")
     k.mfma_attention = False
     try:
-        want = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, D ** -0.5, window)
+        general = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, D ** -0.5, window)
     finally:
         k.mfma_attention = True
-    _close(got, want, torch.bfloat16, "matrix-core kernels against the general kernel")
+    _close(general, want, torch.bfloat16, "general kernel against the float softmax over gathered keys")
     k.check_faults()
 
 

@@ -104,3 +104,16 @@ def test_layer_sizes_of_the_8b_shape(tmp_path, dtype):
         got = H.run_portions(r, "x", toks, portions)
         assert H.rel_err(got, want) < tol, portions
     r.kernels.check_faults()
+    del r
+    # several requests in one step at these sizes: single tokens of three beside a portion of a
+    # fourth, pages of 256, on a pool that holds three of the five requests
+    lens = [300, 270, 40, 290, 180]
+    reqs = {f"r{i}": H.random_tokens(2048, m, 20 + i) for i, m in enumerate(lens)}
+    r = ModelRunner.from_folder(folder, dtype=dtype, page_size=256, num_pages=5, max_requests=4, quiet=True,
+                                enable_prefix_caching=False)
+    got = H.run_mixed(r, reqs, seed=9)
+    for rid, t in reqs.items():
+        want = plain.logits(w, pcfg, t, None if dtype == "float32" else "bfloat16")
+        assert H.rel_err(got[rid], want) < tol, rid
+    assert r.cache.pools[0].num_free == 5
+    r.kernels.check_faults()
