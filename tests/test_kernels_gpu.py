@@ -213,6 +213,18 @@ def test_the_kernel_for_medium_row_counts_in_every_form(hip, m, n, k, splits, ro
         kern.medium_row_tiles, kern.medium_target_workgroups = old
 
 
+def test_rotation_refuses_a_position_beyond_its_table(hip, ref):
+    from nano_vllm_amd.kernels import KernelError
+    k = hip[torch.float32]
+    table = ref.rotary_table(_inv_freq(16, 1e4), 100)
+    qkv = _rand((2, 4 * 16), torch.float32, 1)
+    positions = torch.tensor([3, 100], dtype=torch.int32, device=DEV)
+    with pytest.raises(KernelError, match="no row in the rotary table of 100"):
+        k.qk_norm_rope_store(qkv, 2, 1, 16, None, None, 1e-6, table, positions, None, None, None, max_position=101)
+    with pytest.raises(KernelError, match="needs max_position"):
+        k.qk_norm_rope_store(qkv, 2, 1, 16, None, None, 1e-6, table, positions, None, None, None)
+
+
 def test_split_products_are_consumed_by_norm_and_qk_kernels(hip, ref):
     """A product left as partial sums gives, through the kernels that take it, bit for bit what the
     finished product gives."""
@@ -245,8 +257,8 @@ def test_split_products_are_consumed_by_norm_and_qk_kernels(hip, ref):
     slots = torch.tensor([17, 2, 40, -1, 33], dtype=torch.int32, device=DEV)
     qn, kn = _rand((D,), torch.bfloat16, 36) + 1, _rand((D,), torch.bfloat16, 37) + 1
     caches = [new_caches(4, hkv, D, page, torch.bfloat16, DEV) for _ in range(2)]
-    q1 = k.qk_norm_rope_store(qkv, hq, hkv, D, qn, kn, 1e-6, table, positions, slots, *caches[0])
-    q2 = k.qk_norm_rope_store(full, hq, hkv, D, qn, kn, 1e-6, table, positions, slots, *caches[1])
+    q1 = k.qk_norm_rope_store(qkv, hq, hkv, D, qn, kn, 1e-6, table, positions, slots, *caches[0], max_position=int(positions.max()) + 1)
+    q2 = k.qk_norm_rope_store(full, hq, hkv, D, qn, kn, 1e-6, table, positions, slots, *caches[1], max_position=int(positions.max()) + 1)
     assert torch.equal(q1, q2) and torch.equal(caches[0][0], caches[1][0]) and torch.equal(caches[0][1], caches[1][1])
     assert float(caches[0][1].abs().sum()) > 0
     # the same for a product of more rows, which the kernel for medium row counts leaves
@@ -288,8 +300,8 @@ def test_qk_norm_rope_store(hip, ref, dtype, hq, hkv, D, page, norm):
     slots[5] = -1                                                   # this token is not stored
     caches = [new_caches(pages, hkv, D, page, dtype, DEV) for _ in range(2)]
     a, b = qkv.clone(), qkv.clone()
-    qa = k.qk_norm_rope_store(a, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[0])
-    qb = ref.qk_norm_rope_store(b, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[1])
+    qa = k.qk_norm_rope_store(a, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[0], max_position=int(positions.max()) + 1)
+    qb = ref.qk_norm_rope_store(b, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[1], max_position=int(positions.max()) + 1)
     _close(qa, qb, dtype, "q")
     _close(a, b, dtype, "k in place")
     _close(caches[0][0], caches[1][0], dtype, "k cache")
@@ -325,8 +337,8 @@ def test_qk_norm_rope_store_of_a_long_portion(hip, ref, dtype, hq, hkv, D, page)
     assert len(set(slots.tolist()) - {-1}) == T - 2
     caches = [new_caches(pages, hkv, D, page, dtype, DEV) for _ in range(2)]
     a, b = qkv.clone(), qkv.clone()
-    qa = k.qk_norm_rope_store(a, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[0])
-    qb = ref.qk_norm_rope_store(b, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[1])
+    qa = k.qk_norm_rope_store(a, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[0], max_position=int(positions.max()) + 1)
+    qb = ref.qk_norm_rope_store(b, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[1], max_position=int(positions.max()) + 1)
     _close(qa, qb, dtype, "q")
     _close(a, b, dtype, "k in place")
     _close(caches[0][0], caches[1][0], dtype, "k cache")
