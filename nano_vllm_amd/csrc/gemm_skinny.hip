@@ -14,6 +14,8 @@
 // Requires K % 8 == 0 and 16-byte aligned rows; the launcher refuses anything else and the caller
 // uses the library product or the tiled kernel.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 #include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -531,6 +533,69 @@ NVA_EXPORT int nva_linear_skinny_finish_bf16(const float* partial, int splits, c
     hipLaunchKernelGGL(linear_skinny_finish_kernel, dim3((unsigned)((outs + 255) / 256)), dim3(256), 0, stream, partial,
                        splits, (const __bf16*)bias, y, y_stride, y_is_f32, swiglu, (int)M, (int)N);
     return nva_check_launch("linear_skinny_finish");
+}
+
+// ---------------------------------------------------------------------------- without allocation
+// The partial sums of nva_linear_skinny_static live here (no_alloc.h).  In host code the array's
+// name is a stand-in, not a device address: the address on each device is asked for once, with that
+// device current, and only that pointer is handed to kernels.
+static __device__ __align__(256) float scratch[NVA_STATIC_SCRATCH_FLOATS];
+
+#define NVA_MAX_DEVICES 64
+static float* static_scratch_ptr[NVA_MAX_DEVICES];
+static std::mutex static_scratch_lock;
+
+// The current device's copy of the array, or null after leaving a message.
+static float* static_scratch() {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= NVA_MAX_DEVICES) {
+        nva_fail("linear_skinny_static: no current device (%s)", hipGetErrorString(e));
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> hold(static_scratch_lock);
+    if (!static_scratch_ptr[dev]) {
+        float* ptr = nullptr;
+        e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            nva_fail("linear_skinny_static: the address of the static scratch array on device %d is not to be had (%s)",
+                     dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        static_scratch_ptr[dev] = ptr;
+    }
+    return static_scratch_ptr[dev];
+}
+
+static int skinny_real_splits(int splits, int64_t K) {
+    int kps = (int)((K + splits - 1) / splits);
+    kps = (kps + SK_KSTEP * SK_UNROLL - 1) / (SK_KSTEP * SK_UNROLL) * (SK_KSTEP * SK_UNROLL);
+    return (int)((K + kps - 1) / kps);
+}
+
+NVA_EXPORT int64_t nva_linear_skinny_static_need_bf16(const void* bias, int swiglu, int splits, int64_t M, int64_t N,
+                                                      int64_t K) {
+    if (splits < 1 || M <= 0 || N <= 0 || K <= 0) return 0;
+    if (splits == 1 && !bias) return 0;                    // the product kernel writes y itself (gated or not)
+    return (int64_t)skinny_real_splits(splits, K) * M * N;
+}
+
+NVA_EXPORT int nva_linear_skinny_static_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
+                                             const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
+                                             int splits, int waves_per_tile, int64_t M, int64_t N, int64_t K,
+                                             int* splits_used, hipStream_t stream) {
+    if (M == 0 || N == 0) return 0;
+    if (M < 0 || N < 0 || K <= 0 || splits < 1 || splits > 65535) return nva_fail("linear_skinny_static: bad sizes");
+    const int64_t need = nva_linear_skinny_static_need_bf16(bias, swiglu, splits, M, N, K);
+    if (need > NVA_STATIC_SCRATCH_FLOATS)
+        return nva_fail("linear_skinny_static: %lld ranges of k x %lld rows x %lld columns need %lld floats of partial "
+                        "sums; the static array holds %lld (16 MiB): fewer ranges, or the entry point with a workspace",
+                        (long long)skinny_real_splits(splits, K), (long long)M, (long long)N, (long long)need,
+                        (long long)NVA_STATIC_SCRATCH_FLOATS);
+    float* ptr = static_scratch();
+    if (!ptr) return -1;
+    return nva_linear_skinny_bf16(x, x_stride, w, w_stride, bias, y, y_stride, y_is_f32, swiglu, ptr, splits,
+                                  waves_per_tile, 0, M, N, K, splits_used, stream);
 }
 
 NVA_DEFINE_LAST_ERROR(nva_gemm_skinny)
