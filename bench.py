@@ -31,13 +31,14 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--layers", type=int, default=36, help="layers to build (the shape has 36)")
+    ap.add_argument("--shape", default="qwen3-8b", help="a named shape of nano_vllm_amd.models.shapes (qwen3-8b, qwen3-14b, qwen3-32b)")
+    ap.add_argument("--layers", type=int, default=None, help="layers to build (default: all the shape has)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=256)
     ap.add_argument("--points", default="1,64", help="further decode batch sizes")
     ap.add_argument("--eager", action="store_true", help="no captured decode graph")
-    ap.add_argument("--burst", type=int, default=8,
-                    help="decode steps in a row without the host in between (the engine's decode_burst; 1: one)")
+    ap.add_argument("--burst", type=int, default=None,
+                    help="decode steps in a row without the host in between (default: the engine's decode_burst; 1: one)")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
 
@@ -49,7 +50,7 @@ def main():
         return 2
 
     import torch
-    from nano_vllm_amd.config import Qwen3Config
+    from nano_vllm_amd.config import EngineConfig, Qwen3Config
     from nano_vllm_amd.engine.batch import StepEntry
     from nano_vllm_amd.engine.runner import ModelRunner
     from nano_vllm_amd.kernels import HipKernels
@@ -59,9 +60,11 @@ def main():
     from nano_vllm_amd.weights import fill_random_
 
     from nano_vllm_amd.models.shapes import shape
-    config_json = shape("qwen3-8b")                      # the benchmark's model: layer sizes of Qwen3-8B
+    config_json = shape(args.shape)                     # the default is the benchmark's model: layer sizes of Qwen3-8B
     full_layers = config_json["num_hidden_layers"]
-    config_json.update(num_hidden_layers=args.layers, torch_dtype=args.dtype)
+    if args.burst is None:
+        args.burst = EngineConfig.decode_burst
+    config_json.update(num_hidden_layers=args.layers or full_layers, torch_dtype=args.dtype)
     cfg = Qwen3Config.from_dict(config_json)
     device = "cuda:0"
     dtype = torch_dtype(args.dtype)
@@ -167,12 +170,15 @@ def main():
 
     value, step_s, step_bytes = results[args.batch]
     achieved = step_bytes / step_s / 1e9
+    shape_name = args.shape.replace("qwen", "Qwen").replace("b", "B") if args.shape.startswith("qwen3-") else args.shape
+    short_dtype = "bf16" if args.dtype == "bfloat16" else "fp32"
     line = {
-        "metric": "decode tok/s @ batch 8, context 4096, Qwen3-8B shape bf16 (also batch 1/64 and prefill tok/s @ 2048 tok)",
+        "metric": f"decode tok/s @ batch {args.batch}, context {args.context}, {shape_name} shape {short_dtype} "
+                  f"(also batch {'/'.join(str(b) for b in points if b != args.batch) or '-'} and prefill tok/s @ {T} tok)",
         "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
-        "config": {"model": "Qwen3-8B shape, random weights", "global_batch": args.batch, "seq_len": args.context,
+        "dtype": short_dtype, "data": "synthetic",
+        "config": {"model": f"{shape_name} shape, random weights", "global_batch": args.batch, "seq_len": args.context,
                    "parallelism": "single GPU", "layers": L, "layers_of_shape": full_layers, "hidden_size": H,
                    "num_attention_heads": Hq, "num_key_value_heads": Hkv, "head_dim": D, "intermediate_size": I,
                    "vocab_size": V, "kv_page_size": page, "prefill_tokens": T, "rope_theta": cfg.rope_theta,

@@ -113,21 +113,45 @@ class CacheManager:
             return 0
         return max(0, first_query - w + 1) // self.page_size
 
-    def pages_needed(self, request: Hashable, new_len: int, first_query: Optional[int] = None) -> List[int]:
+    def _wanted_pages(self, group: int, new_len: int, step_end: Optional[int]) -> int:
+        """The length of the group's block table that covers positions < new_len; a window group
+        covers only positions < step_end, the end of the step at hand, when that is given."""
+        if step_end is not None and self.groups[group].window is not None:
+            new_len = min(new_len, step_end)
+        return (new_len + self.page_size - 1) // self.page_size
+
+    def pages_needed(self, request: Hashable, new_len: int, first_query: Optional[int] = None,
+                     step_end: Optional[int] = None) -> List[int]:
         """Per group: the pages that must be taken so that positions < new_len are covered,
         for a step whose first query stands at position first_query (default: the first
-        position not yet reserved)."""
+        position not yet reserved).  With step_end, the end of that step, a window group takes
+        pages up to there only: the pages further on are taken by the steps that reach them,
+        when the window has passed earlier ones."""
         rc = self.requests[request]
         first_query = rc.num_tokens if first_query is None else first_query
-        want = (new_len + self.page_size - 1) // self.page_size
         out = []
         for g, table in enumerate(rc.tables):
             lo = max(len(table), self._first_needed_page(g, first_query))
-            out.append(max(0, want - lo))
+            out.append(max(0, self._wanted_pages(g, new_len, step_end) - lo))
         return out
 
-    def can_reserve(self, request: Hashable, new_len: int, first_query: Optional[int] = None) -> bool:
-        need = self.pages_needed(request, new_len, first_query)
+    def peak_pages(self, num_tokens: int, portion: int) -> List[int]:
+        """Per group: the most pages a request of num_tokens positions holds at any time when no
+        step brings more than `portion` of its tokens.  The all-keys group holds every page; a
+        window group holds those of one step's tokens and of the window before the first of them."""
+        total = (num_tokens + self.page_size - 1) // self.page_size
+        out = []
+        for group in self.groups:
+            if group.window is None:
+                out.append(total)
+            else:
+                span = group.window - 1 + max(1, min(portion, num_tokens))       # positions a step touches, at any offset
+                out.append(min(total, (span + self.page_size - 2) // self.page_size + 1))
+        return out
+
+    def can_reserve(self, request: Hashable, new_len: int, first_query: Optional[int] = None,
+                    step_end: Optional[int] = None) -> bool:
+        need = self.pages_needed(request, new_len, first_query, step_end)
         give = self._passed_pages(request, first_query)
         return all(pool.num_free + g >= n for pool, n, g in zip(self.pools, need, give))
 
@@ -151,16 +175,18 @@ class CacheManager:
             out.append(sum(1 for p in table[:upto] if p >= 0 and self.pools[g].ref_count[p] == 1))
         return out
 
-    def reserve(self, request: Hashable, new_len: int, first_query: Optional[int] = None) -> None:
-        """Makes the block tables cover positions < new_len.  Pages that the window has
-        passed (every position before first_query - window + 1) are given back first.
-        Raises OutOfPages, leaving the request as it was, if a pool cannot give enough."""
+    def reserve(self, request: Hashable, new_len: int, first_query: Optional[int] = None,
+                step_end: Optional[int] = None) -> None:
+        """Makes the block tables cover positions < new_len (a window group: < step_end, if
+        given).  Pages that the window has passed (every position before first_query - window
+        + 1) are given back first.  Raises OutOfPages, leaving the request as it was, if a
+        pool cannot give enough."""
         rc = self.requests[request]
         first_query = rc.num_tokens if first_query is None else first_query
-        if not self.can_reserve(request, new_len, first_query):
+        if not self.can_reserve(request, new_len, first_query, step_end):
             raise OutOfPages(f"request {request!r}: not enough free pages for {new_len} tokens")
-        want = (new_len + self.page_size - 1) // self.page_size
         for g, (pool, table) in enumerate(zip(self.pools, rc.tables)):
+            want = self._wanted_pages(g, new_len, step_end)
             first_page = self._first_needed_page(g, first_query)
             for i in range(min(first_page, len(table))):
                 if table[i] >= 0:
@@ -168,6 +194,8 @@ class CacheManager:
                     table[i] = -1
             while len(table) < want:
                 table.append(pool.take() if len(table) >= first_page else -1)
+        if step_end is not None and any(group.window is not None for group in self.groups):
+            new_len = min(new_len, step_end)                    # positions that every group covers
         rc.num_tokens = max(rc.num_tokens, new_len)
 
     # ------------------------------------------------------------------ prefix reuse
@@ -190,14 +218,15 @@ class CacheManager:
             pages.append(page)
         return len(pages), pages
 
-    def can_admit(self, tokens: Sequence[int]) -> int:
+    def can_admit(self, tokens: Sequence[int], first_step: Optional[int] = None) -> int:
         """-1 if the pages for all of `tokens` are not free, else the number of leading pages
         found in the cache (block_manager.py:58-73): a hit on a page in use costs no free
-        page, a hit on a free page still takes it off the free list."""
+        page, a hit on a free page still takes it off the free list.  A window group needs the
+        pages of the first step's tokens only (first_step of them, default all)."""
         hits, pages = self.match_prefix(tokens)
-        want = (len(tokens) + self.page_size - 1) // self.page_size
+        step_end = None if first_step is None else hits * self.page_size + first_step
         for g, pool in enumerate(self.pools):
-            need = want
+            need = self._wanted_pages(g, len(tokens), step_end)
             if g == 0:
                 need -= sum(1 for p in pages if not pool.is_free(p))
             if pool.num_free < need:
@@ -206,9 +235,10 @@ class CacheManager:
             return -1
         return hits
 
-    def admit_with_prefix(self, request: Hashable, tokens: Sequence[int]) -> int:
+    def admit_with_prefix(self, request: Hashable, tokens: Sequence[int], first_step: Optional[int] = None) -> int:
         """Admits a request, shares the cached leading pages of `tokens` and reserves the
-        rest (block_manager.py:75-92).  Returns the number of tokens already in the cache."""
+        rest (block_manager.py:75-92); a window group reserves the first step's tokens only
+        (first_step of them, default all).  Returns the number of tokens already in the cache."""
         hits, pages = self.match_prefix(tokens)
         rc = self.admit(request)
         try:
@@ -221,7 +251,8 @@ class CacheManager:
                 rc.hashes.append(h)
             cached = hits * self.page_size
             rc.num_tokens = cached
-            self.reserve(request, len(tokens), first_query=cached)
+            self.reserve(request, len(tokens), first_query=cached,
+                         step_end=None if first_step is None else cached + first_step)
         except Exception:
             self.release(request)
             raise

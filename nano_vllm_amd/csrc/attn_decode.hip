@@ -63,8 +63,8 @@ __device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf1
     for (int dt = 0; dt < DT; ++dt) vf[dt] = *reinterpret_cast<const bf16x8*>(pv + (int64_t)dt * 16 * vt);
 }
 
-// waves the GPU holds at once: the kernel's registers allow two per SIMD, eight per CU, on 256 CUs
-#define DEC_RESIDENT_WAVES 2048
+// waves a CU holds at once: the kernel's registers allow two per SIMD, eight per CU
+#define DEC_WAVES_PER_CU 8
 #define DEC_MAX_TOKENS 1024        // tokens of one launch: one wave plans them, 16 to a lane
 
 // The plan of a step's decode attention, made on the device from the tokens' positions by one small
@@ -487,6 +487,21 @@ attn_decode_merge_wave_kernel(const float* __restrict__ part_o, const float* __r
     }
 }
 
+// Waves the current GPU holds at once (asked of the device once), or 0 after leaving a message.
+static int decode_resident_waves() {
+    static int resident = 0;
+    if (!resident) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+            nva_fail("attn_decode: cannot read the number of CUs");
+            return 0;
+        }
+        resident = DEC_WAVES_PER_CU * cus;
+    }
+    return resident;
+}
+
 // What the decode attention of `tokens` single tokens needs when no request holds more than `longest`
 // keys: the bound of the segments of all tokens together, the number of persistent waves (a multiple
 // of the kv heads), and the size of the plan (int32).  Partial results: max_segments * num_q_heads *
@@ -498,7 +513,9 @@ NVA_EXPORT int nva_attn_decode_plan_size_bf16(int longest, int64_t tokens, int n
         return nva_fail("attn_decode_plan_size: bad arguments (at most %d tokens a launch)", DEC_MAX_TOKENS);
     // a token sees at most longest / 32 + 2 chunks (a window may begin and end inside a chunk)
     const int64_t chunks = tokens * ((int64_t)longest / DEC_CHUNK + 2);
-    int64_t per_head = DEC_RESIDENT_WAVES / num_kv_heads > 0 ? DEC_RESIDENT_WAVES / num_kv_heads : 1;
+    const int resident = decode_resident_waves();
+    if (!resident) return -1;
+    int64_t per_head = resident / num_kv_heads > 0 ? resident / num_kv_heads : 1;
     if (per_head > (chunks + 1) / 2) per_head = (chunks + 1) / 2;           // a quota has at least two chunks
     const int64_t cap = decode_quota_cap(page_size);
     const int64_t quotas = per_head > (chunks + cap - 1) / cap ? per_head : (chunks + cap - 1) / cap;
@@ -570,7 +587,9 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     int rc = nva_check_launch("attn_decode");
     if (rc) return rc;
     const int64_t pairs = tokens * num_q_heads;
-    if (pairs >= 2 * DEC_RESIDENT_WAVES) {            // pairs enough for a wave each
+    const int resident = decode_resident_waves();
+    if (!resident) return -1;
+    if (pairs >= 2 * resident) {            // pairs enough for a wave each
         hipLaunchKernelGGL(attn_decode_merge_wave_kernel, dim3((unsigned)((pairs + MERGE_WAVES - 1) / MERGE_WAVES)),
                            dim3(MERGE_WAVES * NVA_WAVE), 0, stream, part_o, part_ml, plan, (__bf16*)out, out_stride,
                            (int)tokens, num_q_heads, head_dim);

@@ -54,10 +54,12 @@ class Scheduler:
         if seq.num_tokens >= self.max_model_len:
             raise ValueError(f"a prompt of {seq.num_tokens} tokens leaves no room below max_model_len "
                              f"{self.max_model_len}")
-        pages = (seq.num_tokens + self.page_size) // self.page_size        # the prompt and one more token
-        smallest = min(pool.num_pages for pool in self.cache.pools) if self.cache.pools else pages
-        if pages > smallest:
-            raise ValueError(f"a prompt of {seq.num_tokens} tokens needs {pages} pages; the cache has {smallest}")
+        # the prompt and one more token, group by group: a window group never holds the whole prompt
+        need = self.cache.peak_pages(seq.num_tokens + 1, self.max_num_batched_tokens)
+        for g, (pages, pool) in enumerate(zip(need, self.cache.pools)):
+            if pages > pool.num_pages:
+                raise ValueError(f"a prompt of {seq.num_tokens} tokens needs {pages} pages of cache group {g}; "
+                                 f"it has {pool.num_pages}")
         self.waiting.append(seq)
 
     # ------------------------------------------------------------------ one step's decision
@@ -78,7 +80,9 @@ class Scheduler:
         while self.waiting and len(batch) < self.max_num_seqs and budget > 0:
             seq = self.waiting[0]
             if not seq.admitted:
-                hits = self.cache.can_admit(seq.token_ids)
+                # all keys: every page of the prompt at admission, as the reference does; a window
+                # group takes the pages of each portion when its step comes
+                hits = self.cache.can_admit(seq.token_ids, budget)
                 if hits == -1:
                     break
                 todo = seq.num_tokens - hits * self.page_size
@@ -87,8 +91,13 @@ class Scheduler:
             if budget < todo and len(batch) > first_here:       # only the first prompt of a step is cut
                 break
             if not seq.admitted:
-                seq.num_cached_tokens = self.cache.admit_with_prefix(seq.seq_id, seq.token_ids)
+                seq.num_cached_tokens = self.cache.admit_with_prefix(seq.seq_id, seq.token_ids, budget)
                 seq.admitted = True
+            else:
+                end = seq.num_cached_tokens + min(todo, budget)
+                if not self.cache.can_reserve(seq.seq_id, seq.num_tokens, seq.num_cached_tokens, step_end=end):
+                    break                                       # a window group waits for pages of running requests
+                self.cache.reserve(seq.seq_id, seq.num_tokens, seq.num_cached_tokens, step_end=end)
             seq.num_scheduled_tokens = min(todo, budget)
             budget -= seq.num_scheduled_tokens
             if seq.num_cached_tokens + seq.num_scheduled_tokens == seq.num_tokens:

@@ -2,7 +2,8 @@
 
 Reference for the whole: nanovllm/models/qwen3.py:162-216 (embedding, the layers in order,
 final norm, output head with optionally tied embedding).  Here the layers and their order
-are data: Model knows no architecture.
+are data, and embedding and head are parts chosen by kind like the others (a scaled embedding
+or a head with a cap on its logits is another kind, registered): Model knows no architecture.
 """
 from __future__ import annotations
 
@@ -35,36 +36,6 @@ class LayerCache:
     state: Optional[Dict[str, torch.Tensor]] = None
 
 
-class TokenEmbedding(Part):
-    """weight [vocab, hidden]; rows are gathered by token id (embed_head.py:24,38)."""
-
-    def __init__(self, params: Mapping, build: BuildContext):
-        super().__init__(params, build)
-        self.vocab, self.hidden = int(params["vocab_size"]), int(params["hidden_size"])
-
-    def param_decls(self):
-        return {"weight": ParamDecl((self.vocab, self.hidden))}
-
-    def forward(self, ids):
-        return self.kernels.embedding(self.weights["weight"], ids)
-
-
-class OutputHead(Part):
-    """logits = x W^T in float32, W [vocab, hidden] (embed_head.py:61); tied: W is the
-    embedding's storage and the checkpoint holds no tensor for it (qwen3.py:202-203)."""
-
-    def __init__(self, params: Mapping, build: BuildContext):
-        super().__init__(params, build)
-        self.vocab, self.hidden = int(params["vocab_size"]), int(params["hidden_size"])
-        self.tied = bool(params.get("tied", False))
-
-    def param_decls(self):
-        return {} if self.tied else {"weight": ParamDecl((self.vocab, self.hidden))}
-
-    def forward(self, x):
-        return self.kernels.linear(x, self.weights["weight"], out_float32=True)
-
-
 class Model:
     def __init__(self, spec: ModelSpec, kernels, device="cuda:0", dtype: Optional[torch.dtype] = None):
         spec.validate()
@@ -77,13 +48,13 @@ class Model:
             build.position_encodings[name] = make_part("position_encoding", pe, build)
         self.position_encodings = build.position_encodings
         sizes = {"vocab_size": spec.vocab_size, "hidden_size": spec.hidden_size}
-        self.embedding = TokenEmbedding({**spec.embedding.params, **sizes}, build)
+        self.embedding = make_part("embedding", PartSpec(spec.embedding.kind, {**spec.embedding.params, **sizes}), build)
         self.blocks: List[Part] = []
         for layer in spec.layers:
             block_spec = PartSpec(layer.block.kind, {**layer.block.params, "parts": layer.parts, "names": layer.names})
             self.blocks.append(make_part("block", block_spec, build))
         self.final_norm = make_part("norm", spec.final_norm, build)
-        self.head = OutputHead({**spec.head.params, **sizes}, build)
+        self.head = make_part("head", PartSpec(spec.head.kind, {**spec.head.params, **sizes}), build)
         self.order: Tuple[LayerRun, ...] = spec.order
 
         # full parameter name -> (owner part, local name, declaration)
@@ -110,7 +81,7 @@ class Model:
         missing = [n for n in self.param_table if n not in self.params]
         if missing:
             raise ValueError(f"parameters without a tensor: {missing}")
-        if self.head.tied:
+        if getattr(self.head, "tied", False):
             self.head.weights["weight"] = self.embedding.weights["weight"]
 
     def num_parameters(self) -> int:

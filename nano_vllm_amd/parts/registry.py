@@ -6,7 +6,7 @@ from __future__ import annotations
 
 from typing import Callable, Dict
 
-ROLES = ("mixer", "feed_forward", "norm", "position_encoding", "block")
+ROLES = ("mixer", "feed_forward", "norm", "position_encoding", "block", "embedding", "head")
 
 _REGISTRIES: Dict[str, Dict[str, Callable]] = {role: {} for role in ROLES}
 
@@ -35,4 +35,4 @@ def known_parts(role: str):
 
 
 def _load_builtin() -> None:
-    from . import norm, rotary, attention, feed_forward, block  # noqa: F401
+    from . import norm, rotary, attention, feed_forward, block, embedding  # noqa: F401

@@ -82,7 +82,7 @@ def load_weights(model, folder: str) -> None:
     if not files:
         raise WeightError(other=[f"{folder!r} holds no *.safetensors file"])
     layout = checkpoint_layout(model)
-    tied_head = model.spec.head["name"] + ".weight" if model.head.tied else None
+    tied_head = model.spec.head["name"] + ".weight" if getattr(model.head, "tied", False) else None
     seen, unexpected, wrong = set(), [], []
     tensors: Dict[str, torch.Tensor] = {}
     tied_copy = None

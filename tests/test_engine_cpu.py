@@ -2,6 +2,8 @@
 on the CPU: the device operations are replaced by their plain torch versions
 (tests/torch_kernels.py), the model and everything above it is the product's.  Compared
 with the plain implementation in float32."""
+import json
+
 import pytest
 import torch
 
@@ -254,3 +256,68 @@ def test_requests_that_share_prefix_pages_give_the_plain_logits(name):
     r = H.make_runner(folder, "float32", c["page"], H.prefix_pool_pages(name, top), device="cpu",
                       kernels=TorchKernels(), prefix_caching=True)
     H.check_prefix_reuse(r, name, top, lambda toks: H.plain_logits(folder, toks), TOL)
+
+
+def test_another_embedding_and_head_are_registered_not_edited_in(tmp_path):
+    """Embedding and head are parts chosen by kind: an embedding that scales its rows and a head
+    that caps its logits are registered here and run through Model.forward unchanged.  Checked
+    against the package's own kinds: the scaled embedding on a table equals the plain embedding
+    on the table times the scale, and the capped logits are cap * tanh(logits / cap)."""
+    import dataclasses
+    import os
+    from safetensors.torch import load_file, save_file
+    from nano_vllm_amd.config.registry import register_architecture
+    from nano_vllm_amd.models.qwen3 import build_spec
+    from nano_vllm_amd.parts import PartSpec, register_part
+    from nano_vllm_amd.parts.embedding import OutputHead, TokenEmbedding
+    from nano_vllm_amd.weights import write_random_model
+
+    scale, cap = 3.0, 0.05
+
+    class ScaledEmbedding(TokenEmbedding):
+        def forward(self, ids):
+            return super().forward(ids) * float(self.params["scale"])
+
+    class CappedHead(OutputHead):
+        def forward(self, x):
+            c = float(self.params["cap"])
+            return torch.tanh(super().forward(x) / c) * c
+
+    def toy_spec(cfg):
+        s = build_spec(cfg)
+        return dataclasses.replace(
+            s, embedding=PartSpec("toy_scaled_embedding", {**s.embedding.params, "scale": scale}),
+            head=PartSpec("toy_capped_head", {**s.head.params, "cap": cap}))
+
+    register_part("embedding", "toy_scaled_embedding", ScaledEmbedding, replace=True)
+    register_part("head", "toy_capped_head", CappedHead, replace=True)
+    register_architecture("ToyScaledCappedLM", H.CONFIGS["b"]["cfg"].from_dict, toy_spec, replace=True)
+
+    base = str(tmp_path / "base")
+    write_random_model(base, H.CONFIGS["b"]["cfg"], seed=5, norm_std=0.1, dtype="float32")
+    tensors = load_file(os.path.join(base, "model.safetensors"))
+    with open(os.path.join(base, "config.json")) as f:
+        cfg_json = json.load(f)
+    # the toy architecture on the same tensors
+    toy = str(tmp_path / "toy")
+    os.makedirs(toy)
+    save_file(tensors, os.path.join(toy, "model.safetensors"), metadata={"format": "pt"})
+    with open(os.path.join(toy, "config.json"), "w") as f:
+        json.dump({**cfg_json, "architectures": ["ToyScaledCappedLM"]}, f)
+    # the package's own kinds on a table that is already scaled
+    scaled = str(tmp_path / "scaled")
+    os.makedirs(scaled)
+    save_file({k: t * scale if k == "model.embed_tokens.weight" else t for k, t in tensors.items()},
+              os.path.join(scaled, "model.safetensors"), metadata={"format": "pt"})
+    with open(os.path.join(scaled, "config.json"), "w") as f:
+        json.dump(cfg_json, f)
+
+    toks = H.random_tokens(384, 40, 9)
+    runs = {}
+    for name, folder in (("toy", toy), ("scaled", scaled), ("base", base)):
+        r = H.make_runner(folder, "float32", 8, 16, device="cpu", kernels=TorchKernels())
+        runs[name] = H.run_portions(r, "x", toks, [25, 1, 14])
+    want = torch.tanh(runs["scaled"] / cap) * cap
+    assert H.rel_err(runs["toy"], want) < TOL
+    assert H.rel_err(runs["base"], runs["scaled"]) > 1e-2        # the scale moves the logits: the check above can fail
+    assert (runs["scaled"].abs() > cap).any()                    # and so does the cap

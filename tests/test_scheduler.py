@@ -204,3 +204,24 @@ def test_mixed_policy_takes_pages_from_a_prompt_that_is_still_being_cut():
     assert any(sid == b.seq_id and start > 0 for _, batch in log for sid, start, n in batch)
     a2, b2, s2, _ = run("prefill_first", 64)
     assert a.token_ids == a2.token_ids and b.token_ids == b2.token_ids and s2.num_preemptions == 0
+
+
+def test_admission_is_sized_group_by_group():
+    """A window group holds the pages of one step's tokens and of the window before them, never
+    the whole prompt: a prompt longer than that group's pool is admitted and runs to the end, and
+    one that the all-keys group cannot hold is refused with the group named."""
+    groups = [CacheGroup(None, (0,)), CacheGroup(6, (1,))]
+    cache = CacheManager(groups, 4, [16, 4], enable_prefix_caching=False)
+    assert cache.peak_pages(41, 8) == [11, 4]         # 6 - 1 + 8 positions at any offset: 4 pages of 4
+    assert cache.peak_pages(3, 8) == [1, 1]
+    s = Scheduler(cache, 4, 8, 64, (), "prefill_first")
+    q = _seq(40)
+    s.add(q)                                          # 11 pages of all keys; the window group has 4 in all
+    _run(s)
+    assert q.is_finished and q.num_completion_tokens == 4
+    assert cache.pools[0].num_free == 16 and cache.pools[1].num_free == 4
+    small = Scheduler(CacheManager(groups, 4, [16, 3], enable_prefix_caching=False), 4, 8, 64, (), "prefill_first")
+    with pytest.raises(ValueError, match="cache group 1"):
+        small.add(_seq(40))
+    with pytest.raises(ValueError, match="cache group 0"):
+        Scheduler(CacheManager(groups, 4, [8, 4], enable_prefix_caching=False), 4, 8, 64, (), "prefill_first").add(_seq(40))
