@@ -21,7 +21,7 @@ _LAST_ERROR_SYMBOL = {
     "activation": "nva_activation_last_error", "rope": "nva_rope_last_error",
     "attn_generic": "nva_attn_generic_last_error", "gemm": "nva_gemm_last_error",
     "sample": "nva_sample_last_error", "attn_decode": "nva_attn_decode_last_error",
-    "gemm_skinny": "nva_gemm_skinny_last_error",
+    "gemm_skinny": "nva_gemm_skinny_last_error", "gemm_team": "nva_gemm_team_last_error",
     "attn_prefill": "nva_attn_prefill_last_error",
 }
 

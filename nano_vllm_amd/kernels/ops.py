@@ -140,6 +140,9 @@ class HipKernels:
         self.medium_max_weight_rows = 8192  # and the widest weight it is used for
         self.medium_row_tiles = 2           # blocks of 16 weight rows per wave in the kernel for up to 128 rows
         self.medium_target_workgroups = 256 # its k range is split until about this many workgroups run (one per CU)
+        self.team_max_rows = 16             # rows of x of the kernel whose waves split k inside a workgroup, for wide weights
+        self.team_min_weight_rows = 8192    # the narrowest weight it is used for (qkv of an 8B model; o and down stay split over workgroups)
+        self.teams = torch.cuda.get_device_properties(self.device).multi_processor_count   # one workgroup per CU
         self.skinny_waves_per_tile = 0      # waves of a workgroup that share rows of the weight and split k; 0: by rows of x
         self.skinny_target_waves = 4096     # the k range of a few-row product is split until this many waves run
         self.fuse_split_sums = True         # False: every product is finished by its own pass
@@ -277,6 +280,15 @@ class HipKernels:
         out_dtype = torch.float32 if out_float32 else x.dtype
         if x.dtype == torch.bfloat16 and self._skinny_takes(x, xs, weight, ws, k):
             own = self._own_kernel(m, n, k)
+            if own == "team":
+                # a wide weight and few rows: k is split inside the workgroups, nothing is deferred
+                if out is None:
+                    out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+                om, on, os_ = _rows2d(out, "linear output")
+                if (om, on) != (m, n) or out.dtype != out_dtype:
+                    raise KernelError("linear: output does not match")
+                self._linear_team(x, xs, weight, ws, bias, out, os_, 1 if out_float32 else 0, m, n, k)
+                return out
             if out_float32 and m > self.own_matmul_rows:
                 # logits of many places: the library product with a float result reads the weight
                 # once, where the streaming kernel would read it once per 64 rows
@@ -333,6 +345,8 @@ class HipKernels:
         (gate/up); small wide weights stay with the skinny kernel up to 64 rows."""
         if m <= 0:
             return None
+        if m <= self.team_max_rows and n >= self.team_min_weight_rows and k % 32 == 0:
+            return "team"
         if m <= self.own_matmul_rows:
             return "skinny"
         if m <= self.medium_max_rows and n <= self.medium_max_weight_rows:
@@ -398,11 +412,21 @@ class HipKernels:
             return SplitSum(self, scratch, used.value, m, n, bias)
         return out
 
+    def _linear_team(self, x, xs, weight, ws, bias, out, os_, mode, m, n, k):
+        """The kernel for wide weights and at most 16 rows.  mode: 0 elements, 1 float, 2 gated."""
+        library.call("gemm_team", "bf16", "nva_linear_team", _p(x), c_i64(xs), _p(weight), c_i64(ws), _p(bias), _p(out),
+                     c_i64(os_), c_i32(mode), c_i64(m), c_i64(n), c_i64(k), c_i32(self.teams), self._stream())
+        return out
+
     def linear_silu_mul(self, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
         """silu(x @ Wg.T) * (x @ Wu.T) with weight = [Wg; Wu]."""
         x = _t(x)
         m, k, xs = _rows2d(x, "linear input")
         n, wk, ws = _rows2d(weight, "linear weight")
+        if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
+                self._own_kernel(m, n, k) == "team" and self._skinny_takes(x, xs, weight, ws, k):
+            out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
+            return self._linear_team(x, xs, weight, ws, None, out, n // 2, 2, m, n, k)
         if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
                 self._own_kernel(m, n, k) == "skinny" and self._skinny_takes(x, xs, weight, ws, k):
             out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)

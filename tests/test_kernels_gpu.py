@@ -190,6 +190,48 @@ def test_linear_silu_mul(hip, ref, m, inner, k):
     _close(hip[torch.float32].linear_silu_mul(xf, wf), ref.linear_silu_mul(xf, wf), torch.float32)
 
 
+@pytest.mark.parametrize("teams", [256, 3])
+@pytest.mark.parametrize("m,n,k", [(1, 64, 64), (3, 200, 96), (8, 6144, 4096), (16, 4096, 12288), (5, 1000, 5120),
+                                   (7, 264, 160), (2, 304, 1632), (4, 1000, 25600), (16, 1016, 6144), (9, 2000, 8192),
+                                   (1, 24576, 4096), (11, 72, 17408)])
+def test_the_kernel_for_wide_weights_and_few_rows_in_every_form(m, n, k, teams):
+    """The kernel whose waves split k inside a workgroup, forced for every weight: x kept in
+    registers (several blocks of weight rows a workgroup) and loaded beside the weight (one
+    block, or k beyond the registers), one pass and several over a wave's slice of k, slices
+    that do not divide, more blocks than lie in LDS at once (3 workgroups), element and float
+    results, bias, the SwiGLU gating, strided rows of x; each against a double product."""
+    from nano_vllm_amd.kernels import HipKernels
+    kern = HipKernels(DEV, torch.bfloat16, quiet=True)
+    kern.team_min_weight_rows, kern.teams = 0, teams
+    assert kern._own_kernel(m, n, k) == "team"
+    wide = _rand((m, k + 8), torch.bfloat16, 61)
+    x = wide[:, 8:]                                       # rows 16 bytes off the allocation's start
+    w, b = _rand((n, k), torch.bfloat16, 62, 0.05), _rand((n,), torch.bfloat16, 63)
+    want = x.double() @ w.double().T
+    bound = (x.double().abs() @ w.double().abs().T) * (math.sqrt(k) * 2.0 ** -23) + 1e-30
+    got32 = kern.linear(x, w, out_float32=True)
+    assert bool(((got32.double() - want).abs() <= bound).all())
+    _close(kern.linear(x, w), want.float().to(torch.bfloat16), torch.bfloat16)
+    _close(kern.linear(x, w, b), (want + b.double()).float().to(torch.bfloat16), torch.bfloat16)
+    gu = want.float().to(torch.bfloat16).float()          # the projection is rounded before the gating
+    gated = torch.nn.functional.silu(gu[:, :n // 2]) * gu[:, n // 2:]
+    _close(kern.linear_silu_mul(x, w), gated, torch.bfloat16)
+    # rows beyond m never reach the result: the same rows beside others
+    if m < 16:
+        more = torch.cat([x, _rand((16 - m, k), torch.bfloat16, 64, 30.0)])
+        assert torch.equal(kern.linear(more, w, out_float32=True)[:m], got32)
+    kern.check_faults()
+
+
+def test_the_kernel_for_wide_weights_refuses_what_it_does_not_take():
+    from nano_vllm_amd.kernels import HipKernels
+    kern = HipKernels(DEV, torch.bfloat16, quiet=True)
+    kern.team_min_weight_rows = 0
+    assert kern._own_kernel(17, 9000, 4096) != "team" and kern._own_kernel(4, 9000, 4104) != "team"
+    x, w = _rand((4, 4104), torch.bfloat16, 65), _rand((9000, 4104), torch.bfloat16, 66, 0.05)
+    _close(kern.linear(x, w), (x.double() @ w.double().T).float().to(torch.bfloat16), torch.bfloat16)
+
+
 @pytest.mark.parametrize("row_tiles", [1, 2])
 @pytest.mark.parametrize("m,n,k,splits", [(128, 512, 1024, 1), (70, 200, 264, 2), (17, 4096, 4096, 8), (97, 72, 8, 1),
                                           (256, 512, 1024, 2), (150, 200, 264, 1), (241, 136, 4096, 4)])

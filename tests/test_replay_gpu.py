@@ -56,6 +56,27 @@ def test_one_request(runners, name, dtype, driving):
     r.kernels.check_faults()
 
 
+@pytest.mark.parametrize("name", ["b", "d"])
+def test_decoding_with_the_kernel_for_wide_weights_forced(name):
+    """At the tiny sizes no weight is wide enough for the kernel whose waves split k inside a
+    workgroup, so the decoded tokens of these models never run it; here it takes every product
+    of up to 16 rows (qkv, o, gate/up with the gating, down, the head; widths are multiples of 32
+    in these two configurations)."""
+    dtype = "bfloat16"
+    n = _length(name)
+    toks = H.random_tokens(H.CONFIGS[name]["cfg"].vocab_size, n, 23)
+    want = H.plain_logits(H.model_folder(name, dtype), toks, ROUNDING[dtype])
+    r = H.make_runner(H.model_folder(name, dtype), dtype, H.CONFIGS[name]["page"], 80)
+    r.kernels.team_min_weight_rows = 0
+    seen = []
+    launch = r.kernels._linear_team
+    r.kernels._linear_team = lambda *a: (seen.append(a[7]), launch(*a))[1]
+    got = H.run_portions(r, "x", toks, [n - 40, 9, 5] + [1] * 26)
+    assert H.rel_err(got, want) < TOL[dtype]
+    assert {0, 1, 2} <= set(seen)                   # element, float and gated results all went through it
+    r.kernels.check_faults()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["a", "b", "c", "d", "e"])
 def test_mixed_requests_on_few_pages(runners, name, dtype):
