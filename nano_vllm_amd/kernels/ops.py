@@ -370,7 +370,9 @@ class HipKernels:
         # split k between them inside the workgroup leave fewer partial sums to add
         # (a gate/up product of up to 16 rows: two waves share the rows, which makes waves enough to
         # leave k unsplit, so that the gating happens in the product kernel and no partial sums are written)
-        kw = self.skinny_waves_per_tile or (4 if m <= 4 else 2 if swiglu and bias is None and m <= 16 else 1)
+        # (a long k, as in a down projection: two waves share the rows at every row count up to 16)
+        kw = self.skinny_waves_per_tile or (2 if k >= 8192 and m <= 16 else 4 if m <= 4 else
+                                            2 if swiglu and bias is None and m <= 16 else 1)
         splits = max(1, min((target + tiles * kw - 1) // (tiles * kw), k // 256))
         if swiglu and bias is None and 2 * tiles * kw >= target:
             splits = 1          # wide enough without a split of k: the gating happens in the product kernel
