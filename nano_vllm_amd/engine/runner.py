@@ -81,6 +81,9 @@ class ModelRunner:
             return          # a mixer with host-side state handling cannot be replayed blindly
         if max_len > self.model.spec.max_position:
             raise ValueError(f"decode graphs for {max_len} tokens: the model knows {self.model.spec.max_position} positions")
+        # which product kernel serves which row count of these steps: measured on the model's own weights
+        if self.device.type == "cuda" and hasattr(self.kernels, "choose_products"):
+            self.kernels.choose_products(self.model.params.values(), max_batch)
         self._graph_max_batch = max_batch
         self._graph_max_len = max_len
         self._graph_table_width = (max_len + self.page_size - 1) // self.page_size

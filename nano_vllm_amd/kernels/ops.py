@@ -97,6 +97,7 @@ def check_positions_fit(table: torch.Tensor, head_dim: int, max_position: Option
                           f"positions (max_position_embeddings)")
 
 
+MEDIUM_KERNEL_ROWS = 256    # rows of x that nva_linear_medium takes
 PREFILL_ROWS = 32       # query rows of one workgroup of the prefill attention kernel
 PREFILL_MAX_TABLE = 4096    # pages of a block-table row the prefill attention kernel stages in LDS
 
@@ -145,6 +146,9 @@ class HipKernels:
         self.teams = torch.cuda.get_device_properties(self.device).multi_processor_count   # one workgroup per CU
         self.skinny_waves_per_tile = 0      # waves of a workgroup that share rows of the weight and split k; 0: by rows of x
         self.skinny_target_waves = 4096     # the k range of a few-row product is split until this many waves run
+        # (n, k, gated) -> {ceil(rows / 16): "library" | "medium" | "skinny"}: what choose_products measured
+        # for the model's own weights; where it has no entry the rules of _own_kernel decide
+        self.product_choice = {}
         self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
         self.mfma_attention = True
@@ -335,25 +339,86 @@ class HipKernels:
                      c_i64(m), c_i64(n), c_i64(k), self._stream())
         return out
 
-    def _own_kernel(self, m: int, n: int, k: int) -> Optional[str]:
+    def _own_kernel(self, m: int, n: int, k: int, gated: bool = False) -> Optional[str]:
         """Which of the engine's weight-streaming kernels takes a bfloat16 product of m rows with a
-        weight [n, k]: "skinny", "medium", or None for the library product.  Measured on the layer
-        shapes of an 8B model: up to 16 rows the skinny kernel is as fast or faster for every
-        weight; up to 224 rows the medium kernel wins for weights of few rows (the library has no
-        split of k and leaves most of the GPU idle there: o and down projections take twice as
-        long; at 256 rows the library's tiles fit and it draws level), and loses for wide ones
-        (gate/up); small wide weights stay with the skinny kernel up to 64 rows."""
+        weight [n, k]: "team", "skinny", "medium", or None for the library product.  Up to 16 rows
+        the engine's own kernels are as fast or faster for every weight ("team" for wide weights,
+        whose waves split k inside a workgroup; "skinny" otherwise).  Beyond that the answer
+        depends on the weight's shape and on what the library's heuristics pick for it, so it is
+        measured once for the model's own weights (choose_products); without a measurement the
+        rules below stand, which were measured on the layer shapes of an 8B model: up to 224 rows
+        the medium kernel wins for weights of few rows (the library has no split of k and leaves
+        most of the GPU idle there), and loses for wide ones (gate/up); small wide weights stay
+        with the skinny kernel up to 64 rows."""
         if m <= 0:
             return None
         if m <= self.team_max_rows and n >= self.team_min_weight_rows and k % 32 == 0:
             return "team"
         if m <= self.own_matmul_rows:
             return "skinny"
+        measured = self.product_choice.get((n, k, gated))
+        if measured is not None and (m + 15) // 16 in measured:
+            choice = measured[(m + 15) // 16]
+            return None if choice == "library" else choice
         if m <= self.medium_max_rows and n <= self.medium_max_weight_rows:
             return "medium"
         if m <= self.skinny_max_rows and 2 * n * k <= self.small_weight_bytes:
             return "skinny"
         return None
+
+    def choose_products(self, tensors, max_rows: int, min_elements: int = 1 << 22, reps: int = 3) -> dict:
+        """Measures, for every shape of weight among `tensors` (2-D bfloat16 of at least min_elements
+        elements and at most 65536 rows: the layers' projections) and every row count that a captured
+        decode step of up to max_rows requests can have beyond 16 (multiples of 16, at most 256),
+        the library product against the engine's own kernels, plain (as a norm or the q/k
+        preparation consumes it) and with the SwiGLU gating, and keeps the fastest per shape and
+        row count in self.product_choice.  The weights of one shape (one per layer) are used in
+        turn, so that none is found in a cache.  Returns what it chose."""
+        import torch.nn.functional as F
+        by_shape = {}
+        for t in tensors:
+            if t.dim() == 2 and t.dtype == torch.bfloat16 and t.is_cuda and t.numel() >= min_elements and \
+                    t.shape[0] <= 65536 and t.is_contiguous():
+                by_shape.setdefault(tuple(t.shape), []).append(t)
+        rows = [m for m in range(32, min(max_rows, MEDIUM_KERNEL_ROWS) + 1, 16)]
+        if not by_shape or not rows:
+            return {}
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+        def timed(fn, weights) -> float:
+            fn(weights[0])
+            start.record()
+            for i in range(reps):
+                fn(weights[(i + 1) % len(weights)])
+            stop.record()
+            stop.synchronize()
+            return start.elapsed_time(stop)
+
+        for (n, k), weights in by_shape.items():
+            if not self._skinny_takes(weights[0], k, weights[0], k, k):
+                continue
+            for gated in (False, True):
+                if gated and n % 2:
+                    continue
+                table = {}
+                for m in rows:
+                    x = torch.randn((m, k), dtype=torch.bfloat16, device=weights[0].device)
+                    out = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=x.device)
+                    cands = {}
+                    if gated:
+                        cands["library"] = lambda w: self.silu_mul(F.linear(x, w), out=out)
+                        cands["medium"] = lambda w: self._linear_medium(x, k, w, k, None, out, n // 2, False, True, m, n, k)
+                        if m <= self.skinny_max_rows:
+                            cands["skinny"] = lambda w: self._linear_skinny(x, k, w, k, None, out, n // 2, False, True, m, n, k)
+                    else:
+                        cands["library"] = lambda w: F.linear(x, w)
+                        cands["medium"] = lambda w: self._linear_medium(x, k, w, k, None, None, 0, False, False, m, n, k, defer=True)
+                        if m <= self.skinny_max_rows:
+                            cands["skinny"] = lambda w: self._linear_skinny(x, k, w, k, None, None, 0, False, False, m, n, k, defer=True)
+                    times = {name: timed(fn, weights) for name, fn in cands.items()}
+                    table[m // 16] = min(times, key=times.get)
+                self.product_choice[(n, k, gated)] = table
+        return self.product_choice
 
     @staticmethod
     def _skinny_takes(x, xs, weight, ws, k) -> bool:
@@ -430,10 +495,15 @@ class HipKernels:
             out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
             return self._linear_team(x, xs, weight, ws, None, out, n // 2, 2, m, n, k)
         if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
-                self._own_kernel(m, n, k) == "skinny" and self._skinny_takes(x, xs, weight, ws, k):
-            out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
-            self._linear_skinny(x, xs, weight, ws, None, out, n // 2, False, True, m, n, k)
-            return out
+                self._skinny_takes(x, xs, weight, ws, k):
+            own = self._own_kernel(m, n, k, gated=True)
+            if own in ("skinny", "medium"):
+                out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
+                run = self._linear_skinny if own == "skinny" else self._linear_medium
+                run(x, xs, weight, ws, None, out, n // 2, False, True, m, n, k)
+                return out
+            if m > self.own_matmul_rows and (n, k, True) in self.product_choice:
+                return self.silu_mul(torch.nn.functional.linear(x, weight))      # measured: the library here
         return self.silu_mul(self.linear(x, weight))
 
     # ------------------------------------------------------------------ position encoding
