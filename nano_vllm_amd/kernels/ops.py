@@ -146,7 +146,7 @@ class HipKernels:
         self.teams = torch.cuda.get_device_properties(self.device).multi_processor_count   # one workgroup per CU
         self.skinny_waves_per_tile = 0      # waves of a workgroup that share rows of the weight and split k; 0: by rows of x
         self.skinny_target_waves = 4096     # the k range of a few-row product is split until this many waves run
-        # (n, k, gated) -> {ceil(rows / 16): "library" | "medium" | "skinny"}: what choose_products measured
+        # (n, k, gated) -> {ceil(rows / 16): "library" | "medium"}: what choose_products measured
         # for the model's own weights; where it has no entry the rules of _own_kernel decide
         self.product_choice = {}
         self.fuse_split_sums = True         # False: every product is finished by its own pass
@@ -370,8 +370,8 @@ class HipKernels:
         """Measures, for every shape of weight among `tensors` (2-D bfloat16 of at least min_elements
         elements and at most 65536 rows: the layers' projections) and every row count that a captured
         decode step of up to max_rows requests can have beyond 16 (multiples of 16, at most 256),
-        the library product against the engine's own kernels, plain (as a norm or the q/k
-        preparation consumes it) and with the SwiGLU gating, and keeps the fastest per shape and
+        the library product against the engine's kernel for up to 256 rows, plain (as a norm or the
+        q/k preparation consumes it) and with the SwiGLU gating, and keeps the fastest per shape and
         row count in self.product_choice.  The weights of one shape (one per layer) are used in
         turn, so that none is found in a cache.  Returns what it chose."""
         import torch.nn.functional as F
@@ -408,14 +408,11 @@ class HipKernels:
                     if gated:
                         cands["library"] = lambda w: self.silu_mul(F.linear(x, w), out=out)
                         cands["medium"] = lambda w: self._linear_medium(x, k, w, k, None, out, n // 2, False, True, m, n, k)
-                        if m <= self.skinny_max_rows:
-                            cands["skinny"] = lambda w: self._linear_skinny(x, k, w, k, None, out, n // 2, False, True, m, n, k)
                     else:
                         cands["library"] = lambda w: F.linear(x, w)
                         cands["medium"] = lambda w: self._linear_medium(x, k, w, k, None, None, 0, False, False, m, n, k, defer=True)
-                        if m <= self.skinny_max_rows:
-                            cands["skinny"] = lambda w: self._linear_skinny(x, k, w, k, None, None, 0, False, False, m, n, k, defer=True)
-                    times = {name: timed(fn, weights) for name, fn in cands.items()}
+                    # the smaller of two measurements each: a start-up has other work going on
+                    times = {name: min(timed(fn, weights), timed(fn, weights)) for name, fn in cands.items()}
                     table[m // 16] = min(times, key=times.get)
                 self.product_choice[(n, k, gated)] = table
         return self.product_choice
