@@ -223,6 +223,34 @@ def test_the_kernel_for_wide_weights_and_few_rows_in_every_form(m, n, k, teams):
     kern.check_faults()
 
 
+def test_the_product_kernel_is_chosen_by_measurement_and_every_choice_is_right():
+    """choose_products times the library against the engine's kernel on the given weights and fills
+    a table per (shape, gated) and 16 rows; whatever it chose, and each choice forced, gives the
+    product of a double computation, plain and gated."""
+    from nano_vllm_amd.kernels import HipKernels
+    kern = HipKernels(DEV, torch.bfloat16, quiet=True)
+    n, k = 4096, 1024
+    weights = [_rand((n, k), torch.bfloat16, 70 + i, 0.05) for i in range(3)]
+    small = _rand((64, 64), torch.bfloat16, 75)                     # below min_elements: not measured
+    table = kern.choose_products(weights + [small, weights[0].float()], max_rows=80)
+    assert set(table) == {(n, k, False), (n, k, True)}
+    for gated in (False, True):
+        assert set(table[(n, k, gated)]) == {2, 3, 4, 5} and set(table[(n, k, gated)].values()) <= {"library", "medium"}
+    x = _rand((40, k), torch.bfloat16, 76)
+    want = x.double() @ weights[1].double().T
+    gu = want.float().to(torch.bfloat16).float()
+    gated_want = torch.nn.functional.silu(gu[:, :n // 2]) * gu[:, n // 2:]
+    for forced in (None, "library", "medium"):
+        if forced:
+            kern.product_choice = {(n, k, g): {b: forced for b in range(2, 6)} for g in (False, True)}
+            assert kern._own_kernel(40, n, k) == (None if forced == "library" else forced)
+        _close(kern.linear(x, weights[1]), want.float().to(torch.bfloat16), torch.bfloat16, str(forced))
+        _close(kern.linear_silu_mul(x, weights[1]), gated_want, torch.bfloat16, str(forced))
+        got = kern.linear(x, weights[1], deferred=True)
+        _close(got.tensor() if hasattr(got, "tensor") else got, want.float().to(torch.bfloat16), torch.bfloat16, str(forced))
+    kern.check_faults()
+
+
 def test_the_kernel_for_wide_weights_refuses_what_it_does_not_take():
     from nano_vllm_amd.kernels import HipKernels
     kern = HipKernels(DEV, torch.bfloat16, quiet=True)
