@@ -206,10 +206,12 @@ linear_skinny_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
 // direct and the layout of the results: as above.
 #define MD_KC 128
 #define MD_XS (MD_KC + 8)
-#define MD_WAVES 4
 #define MD_MAX_ROWS 256
-template <int MB, int RT>
-__global__ void __launch_bounds__(MD_WAVES * NVA_WAVE) __attribute__((amdgpu_waves_per_eu(MB > 8 ? 1 : 2)))
+// WAVES (3 or 4) and RT (1 to 3) set how many blocks of 16 weight rows a workgroup takes: a CU draws
+// only about its share of the memory's bandwidth, so the product is as fast as its most loaded CU,
+// and the launcher's caller picks the pair that spreads the weight's blocks evenly over the CUs.
+template <int MB, int RT, int WAVES>
+__global__ void __launch_bounds__(WAVES * NVA_WAVE) __attribute__((amdgpu_waves_per_eu(MB > 8 ? 1 : 2)))
 linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf16* __restrict__ w, int64_t w_stride,
                      float* __restrict__ partial, void* __restrict__ y, int64_t y_stride, int y_is_f32, int direct,
                      int M, int N, int K, int k_per_split) {
@@ -224,7 +226,7 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
     const bool gated = direct == 2;
     const int inner = N / 2;
     const int per_tile = gated ? 8 : 16;
-    const int tile0 = (blockIdx.x * MD_WAVES + wave) * RT;
+    const int tile0 = (blockIdx.x * WAVES + wave) * RT;
     const int k_last = K - 8;
 
     const __bf16* wrow[RT];
@@ -242,8 +244,8 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) acc[rt][b] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    // staging: thread t moves the 16-byte piece t % 16 of rows t / 16 + SR * j
-    constexpr int SR = MD_WAVES * NVA_WAVE / 16, SJ = 16 * MB / SR;
+    // staging: thread t moves the 16-byte piece t % 16 of rows t / 16 + SR * j (below 16 * MB)
+    constexpr int SR = WAVES * NVA_WAVE / 16, SJ = (16 * MB + SR - 1) / SR;
     const int s_row = threadIdx.x / 16, s_piece = threadIdx.x % 16;
     constexpr int XD = MB > 8 ? 1 : 2;                                // chunks that x is asked for ahead (registers allowing)
     bf16x8 xr[XD][SJ];                                                // x of the next chunks, on its way
@@ -260,8 +262,9 @@ linear_medium_kernel(const __bf16* __restrict__ x, int64_t x_stride, const __bf1
         const bool k_ok = k0 + 8 * s_piece < k_end;
 #pragma unroll
         for (int j = 0; j < SJ; ++j)
-            *reinterpret_cast<bf16x8*>(&x_s[(buf * ROWS + s_row + SR * j) * MD_XS + 8 * s_piece]) =
-                k_ok && s_row + SR * j < M ? xr[j] : zero8();
+            if (16 * MB % SR == 0 || s_row + SR * j < 16 * MB)
+                *reinterpret_cast<bf16x8*>(&x_s[(buf * ROWS + s_row + SR * j) * MD_XS + 8 * s_piece]) =
+                    k_ok && s_row + SR * j < M ? xr[j] : zero8();
     };
     // Workgroups walk their chunks in rotated order, each from another start: at one k the rows of
     // x (a power of two apart, as a rule) lie in few channels of the L2, and workgroups that all
@@ -465,12 +468,12 @@ NVA_EXPORT int nva_linear_skinny_bf16(const void* x, int64_t x_stride, const voi
     return nva_check_launch("linear_skinny_finish");
 }
 
-// The kernel for up to 256 rows of x.  row_tiles: 1 or 2 blocks of 16 rows of W per wave (always 1
-// beyond 224 rows).  The other
-// arguments as for nva_linear_skinny; k per range is rounded up to a multiple of 128.
+// The kernel for up to 256 rows of x.  waves (3 or 4; 3 up to 96 rows of x) and row_tiles (1 to 3; 3 up
+// to 96 rows, 1 beyond 224): a workgroup takes waves * row_tiles blocks of 16 rows of W.  The other arguments as for
+// nva_linear_skinny; k per range is rounded up to a multiple of 128.
 NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride,
                                       const void* bias, void* y, int64_t y_stride, int y_is_f32, int swiglu,
-                                      float* scratch, int splits, int row_tiles, int defer_finish, int64_t M,
+                                      float* scratch, int splits, int row_tiles, int waves, int defer_finish, int64_t M,
                                       int64_t N, int64_t K, int* splits_used, hipStream_t stream) {
     if (M == 0 || N == 0) return 0;
     if (M < 0 || M > MD_MAX_ROWS || K % 8 || K <= 0 || x_stride % 8 || w_stride % 8 || !nva_aligned(x, 16) || !nva_aligned(w, 16)) {
@@ -479,7 +482,10 @@ NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const voi
         return 1;
     }
     if (N > 0x7fffffff || K > 0x7fffffff || splits < 1 || splits > 65535) return nva_fail("linear_medium: bad sizes");
-    if (row_tiles != 1 && row_tiles != 2) return nva_fail("linear_medium: 1 or 2 row tiles per wave, not %d", row_tiles);
+    const int mb = (int)((M + 15) / 16 + 1) / 2 * 2;                   // instances for 2, 4, 6, ... 16 blocks of 16 rows
+    if (waves != 3 && waves != 4) return nva_fail("linear_medium: 3 or 4 waves per workgroup, not %d", waves);
+    if (row_tiles < 1 || row_tiles > 3 || (row_tiles == 3 && mb > 6) || (row_tiles == 2 && mb > 14) || (waves == 3 && mb > 6))
+        return nva_fail("linear_medium: %d row tiles per wave and %d waves are not built for %lld rows", row_tiles, waves, (long long)M);
     if (swiglu && (N % 2)) return nva_fail("linear_medium: the gated form needs an even number of weight rows");
     const int direct = splits == 1 && !bias && !defer_finish ? (swiglu ? 2 : 1) : 0;
     if (!direct && !scratch) return nva_fail("linear_medium: this call needs scratch memory");
@@ -487,31 +493,36 @@ NVA_EXPORT int nva_linear_medium_bf16(const void* x, int64_t x_stride, const voi
     kps = (kps + MD_KC - 1) / MD_KC * MD_KC;
     const int real_splits = (int)((K + kps - 1) / kps);
     const int64_t tiles = direct == 2 ? (N / 2 + 7) / 8 : (N + 15) / 16;
-    const int mb = (int)((M + 15) / 16 + 1) / 2 * 2;                   // instances for 2, 4, 6, 8 blocks of 16 rows
     const size_t lds = (size_t)2 * (16 * mb + 1) * MD_XS * sizeof(__bf16);
-#define LAUNCH(MB, RT)                                                                                                 \
+#define LAUNCH(MB, RT, WV)                                                                                             \
     do {                                                                                                               \
-        dim3 grid((unsigned)((tiles + MD_WAVES * RT - 1) / (MD_WAVES * RT)), (unsigned)real_splits);                   \
-        hipLaunchKernelGGL((linear_medium_kernel<MB, RT>), grid, dim3(MD_WAVES * NVA_WAVE), lds, stream,               \
+        dim3 grid((unsigned)((tiles + WV * RT - 1) / (WV * RT)), (unsigned)real_splits);                               \
+        hipLaunchKernelGGL((linear_medium_kernel<MB, RT, WV>), grid, dim3(WV * NVA_WAVE), lds, stream,                 \
                            (const __bf16*)x, x_stride, (const __bf16*)w, w_stride, scratch, y, y_stride, y_is_f32,     \
                            direct, (int)M, (int)N, (int)K, kps);                                                       \
     } while (0)
-#define LAUNCH_RT(MB)                                                                                                  \
+#define LAUNCH_SMALL(MB)                                                                                               \
     do {                                                                                                               \
-        if (row_tiles == 1) LAUNCH(MB, 1);                                                                             \
-        else LAUNCH(MB, 2);                                                                                            \
+        if (waves == 4) { if (row_tiles == 1) LAUNCH(MB, 1, 4); else if (row_tiles == 2) LAUNCH(MB, 2, 4); else LAUNCH(MB, 3, 4); } \
+        else { if (row_tiles == 1) LAUNCH(MB, 1, 3); else if (row_tiles == 2) LAUNCH(MB, 2, 3); else LAUNCH(MB, 3, 3); } \
     } while (0)
-    switch (mb) {                      // more than 224 rows: one block of weight rows per wave (registers)
-        case 2: LAUNCH_RT(2); break;
-        case 4: LAUNCH_RT(4); break;
-        case 6: LAUNCH_RT(6); break;
-        case 8: LAUNCH_RT(8); break;
-        case 10: LAUNCH_RT(10); break;
-        case 12: LAUNCH_RT(12); break;
-        case 14: LAUNCH_RT(14); break;
-        default: LAUNCH(16, 1); break;
+#define LAUNCH_LARGE(MB)                                                                                               \
+    do {                                                                                                               \
+        if (row_tiles == 1) LAUNCH(MB, 1, 4);                                                                          \
+        else LAUNCH(MB, 2, 4);                                                                                         \
+    } while (0)
+    switch (mb) {
+        case 2: LAUNCH_SMALL(2); break;
+        case 4: LAUNCH_SMALL(4); break;
+        case 6: LAUNCH_SMALL(6); break;
+        case 8: LAUNCH_LARGE(8); break;
+        case 10: LAUNCH_LARGE(10); break;
+        case 12: LAUNCH_LARGE(12); break;
+        case 14: LAUNCH_LARGE(14); break;
+        default: LAUNCH(16, 1, 4); break;      // more than 224 rows: one block of weight rows per wave (registers)
     }
-#undef LAUNCH_RT
+#undef LAUNCH_SMALL
+#undef LAUNCH_LARGE
 #undef LAUNCH
     if (splits_used) *splits_used = real_splits;
     int rc = nva_check_launch("linear_medium");

@@ -139,8 +139,9 @@ class HipKernels:
         self.small_weight_bytes = 64 << 20
         self.medium_max_rows = 224          # rows of x the kernel for medium row counts is used for (it takes 256)
         self.medium_max_weight_rows = 8192  # and the widest weight it is used for
-        self.medium_row_tiles = 2           # blocks of 16 weight rows per wave in the kernel for up to 128 rows
-        self.medium_target_workgroups = 256 # its k range is split until about this many workgroups run (one per CU)
+        self.medium_row_tiles = 2           # 1: one block of 16 weight rows per wave in the kernel for up to 256 rows (tests)
+        self.medium_shape = None            # (waves, row tiles, ranges of k) forced on that kernel (tests)
+        self.medium_target_workgroups = torch.cuda.get_device_properties(self.device).multi_processor_count   # one workgroup per CU
         self.team_max_rows = 16             # rows of x of the kernel whose waves split k inside a workgroup, for wide weights
         self.team_min_weight_rows = 8192    # the narrowest weight it is used for (qkv of an 8B model; o and down stay split over workgroups)
         self.teams = torch.cuda.get_device_properties(self.device).multi_processor_count   # one workgroup per CU
@@ -453,14 +454,43 @@ class HipKernels:
             return SplitSum(self, scratch, used.value, m, n, bias)
         return out
 
+    def _medium_shape(self, m: int, blocks: int, k: int):
+        """(waves, row tiles, ranges of k) of the kernel for up to 256 rows, for a weight of `blocks`
+        blocks of 16 rows.  A CU draws about its share of the memory's bandwidth and no more, so the
+        product takes as long as its most loaded CU: of the workgroup sizes the kernel is built with
+        (3 or 4 waves of 1 to 3 blocks each, fewer choices for many rows of x) the one is taken whose
+        workgroups spread most evenly over the CUs; a weight of few blocks takes the largest
+        workgroups and is split over k instead, into as many ranges as give at most one workgroup per
+        CU (a second, partly filled round of workgroups costs more than CUs left idle)."""
+        if self.medium_shape is not None:
+            return self.medium_shape
+        cus = self.medium_target_workgroups
+        mb = ((m + 15) // 16 + 1) // 2 * 2
+        if mb > 14:
+            sizes = [(4, 1)]
+        elif mb > 6:
+            sizes = [(4, 2), (4, 1)]
+        else:
+            sizes = [(4, 2), (3, 3), (4, 3), (3, 2), (4, 1), (3, 1)]
+        if self.medium_row_tiles == 1:
+            sizes = [s for s in sizes if s[1] == 1] or sizes
+        waves, rt = sizes[0]
+        wgs = (blocks + waves * rt - 1) // (waves * rt)
+        if 2 * wgs <= cus:
+            return waves, rt, max(1, min(cus // wgs, k // 256))        # a weight of few blocks: split over k
+        best = None
+        for waves, rt in sizes:
+            wgs = (blocks + waves * rt - 1) // (waves * rt)
+            # rows (of the weight, and of x once per workgroup) that the most loaded CU streams
+            cost = (((wgs + cus - 1) // cus) * (16 * waves * rt + m), -waves * rt)
+            if best is None or cost < best[0]:
+                best = (cost, waves, rt, 1)
+        return best[1], best[2], best[3]
+
     def _linear_medium(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k, defer=False):
         """The weight-streaming kernel for up to 256 rows (see _linear_skinny for the arguments)."""
-        rt = self.medium_row_tiles if m <= 224 else 1      # more rows: the kernel's registers hold one block
-        tiles = (n + 15) // 16
-        wgs = (tiles + 4 * rt - 1) // (4 * rt)
-        # as many ranges of k as give at most one workgroup per CU: a second, partly filled round of
-        # workgroups costs more than CUs left idle
-        splits = max(1, min(self.medium_target_workgroups // wgs, k // 256))
+        blocks = (n // 2 + 7) // 8 if swiglu and bias is None and not defer else (n + 15) // 16
+        waves, rt, splits = self._medium_shape(m, blocks, k)
         if defer and splits == 1:
             defer = False
             out = torch.empty((m, n), dtype=x.dtype, device=x.device)
@@ -470,8 +500,8 @@ class HipKernels:
         used = ctypes.c_int(0)
         library.call("gemm_skinny", "bf16", "nva_linear_medium", _p(x), c_i64(xs), _p(weight), c_i64(ws),
                      None if defer else _p(bias), _p(out), c_i64(os_), c_i32(1 if out_float32 else 0),
-                     c_i32(1 if swiglu else 0), _p(scratch), c_i32(splits), c_i32(rt), c_i32(1 if defer else 0), c_i64(m),
-                     c_i64(n), c_i64(k), ctypes.byref(used), self._stream())
+                     c_i32(1 if swiglu else 0), _p(scratch), c_i32(splits), c_i32(rt), c_i32(waves), c_i32(1 if defer else 0),
+                     c_i64(m), c_i64(n), c_i64(k), ctypes.byref(used), self._stream())
         if defer:
             return SplitSum(self, scratch, used.value, m, n, bias)
         return out

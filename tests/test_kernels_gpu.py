@@ -260,17 +260,29 @@ def test_the_kernel_for_wide_weights_refuses_what_it_does_not_take():
     _close(kern.linear(x, w), (x.double() @ w.double().T).float().to(torch.bfloat16), torch.bfloat16)
 
 
-@pytest.mark.parametrize("row_tiles", [1, 2])
+@pytest.mark.parametrize("waves,row_tiles", [(4, 1), (4, 2), (4, 3), (3, 1), (3, 2), (3, 3)])
 @pytest.mark.parametrize("m,n,k,splits", [(128, 512, 1024, 1), (70, 200, 264, 2), (17, 4096, 4096, 8), (97, 72, 8, 1),
-                                          (256, 512, 1024, 2), (150, 200, 264, 1), (241, 136, 4096, 4)])
-def test_the_kernel_for_medium_row_counts_in_every_form(hip, m, n, k, splits, row_tiles):
-    """Unsplit and split over k, one and two blocks of weight rows per wave, plain and gated."""
+                                          (256, 512, 1024, 2), (150, 200, 264, 1), (241, 136, 4096, 4), (33, 1000, 520, 1),
+                                          (96, 328, 1288, 3), (48, 24, 96, 1)])
+def test_the_kernel_for_medium_row_counts_in_every_form(hip, m, n, k, splits, waves, row_tiles):
+    """Unsplit and split over k, three and four waves of one to three blocks of weight rows each
+    (where the kernel is built with them: up to 96 rows of x all, up to 224 rows four waves of one or
+    two blocks, beyond that of one), plain and gated."""
     kern = hip[torch.bfloat16]
+    blocks_of_x = ((m + 15) // 16 + 1) // 2 * 2
+    if (blocks_of_x > 6 and (waves == 3 or row_tiles == 3)) or (blocks_of_x > 14 and row_tiles == 2):
+        from nano_vllm_amd.kernels import KernelError
+        kern.medium_shape = (waves, row_tiles, 1)
+        try:
+            with pytest.raises(KernelError, match="not built"):
+                kern._linear_medium(_rand((m, k), torch.bfloat16, 41), k, _rand((n, k), torch.bfloat16, 42), k, None,
+                                    torch.empty((m, n), dtype=torch.bfloat16, device=DEV), n, False, False, m, n, k)
+        finally:
+            kern.medium_shape = None
+        return
     x, w = _rand((m, k), torch.bfloat16, 41), _rand((n, k), torch.bfloat16, 42, 0.05)
     want = x.double() @ w.double().T
-    old = kern.medium_row_tiles, kern.medium_target_workgroups
-    kern.medium_row_tiles = row_tiles
-    kern.medium_target_workgroups = splits * ((n + 15) // 16 + 4 * row_tiles - 1) // (4 * row_tiles)
+    kern.medium_shape = (waves, row_tiles, splits)
     try:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
         kern._linear_medium(x, k, w, k, None, out, n, False, False, m, n, k)
@@ -279,8 +291,29 @@ def test_the_kernel_for_medium_row_counts_in_every_form(hip, m, n, k, splits, ro
         kern._linear_medium(x, k, w, k, None, gated, n // 2, False, True, m, n, k)
         y = want.float().to(torch.bfloat16).float()
         _close(gated, (torch.nn.functional.silu(y[:, :n // 2]) * y[:, n // 2:]).to(torch.bfloat16), torch.bfloat16)
+        got = kern._linear_medium(x, k, w, k, None, None, 0, False, False, m, n, k, defer=True)
+        _close(got.tensor() if hasattr(got, "tensor") else got, want.float().to(torch.bfloat16), torch.bfloat16)
     finally:
-        kern.medium_row_tiles, kern.medium_target_workgroups = old
+        kern.medium_shape = None
+    kern.check_faults()
+
+
+def test_the_kernel_for_medium_row_counts_spreads_a_weight_evenly_over_the_cus(hip):
+    """What _medium_shape picks: for the gate/up weight of an 8B model (1536 blocks of 16 rows) six
+    blocks a workgroup, which is one workgroup for each of 256 CUs, not eight (192 workgroups, a
+    quarter of the CUs idle); a weight of few blocks is split over k until every CU has a workgroup."""
+    kern = hip[torch.bfloat16]
+    old = kern.medium_target_workgroups
+    kern.medium_target_workgroups = 256
+    try:
+        waves, rt, splits = kern._medium_shape(64, 1536, 4096)
+        assert waves * rt == 6 and splits == 1
+        waves, rt, splits = kern._medium_shape(64, 256, 4096)
+        assert (256 // (waves * rt)) * splits == 256
+        assert kern._medium_shape(64, 3200, 5120) == (4, 2, 1)      # few large workgroups read x less often than many small
+        assert kern._medium_shape(240, 1536, 4096) == (4, 1, 1) and kern._medium_shape(200, 3200, 5120)[:2] == (4, 2)
+    finally:
+        kern.medium_target_workgroups = old
 
 
 def test_rotation_refuses_a_position_beyond_its_table(hip, ref):
