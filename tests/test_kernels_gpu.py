@@ -459,7 +459,7 @@ def test_qk_refusals(hip):
 
 
 # ------------------------------------------------------------------------------ attention
-def _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed, boost=None):
+def _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed, boost=None, fill=1.0):
     """A batch of requests with kv lengths `lens`, the last q_lens of which are this step's
     queries; keys and values scattered over shuffled pages."""
     rng = random.Random(seed)
@@ -468,7 +468,9 @@ def _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed, boost=None):
     total = sum(pages_per) + 3
     order = list(range(total))
     rng.shuffle(order)
-    kc, vc = new_caches(total, hkv, D, page, dtype, DEV, fill=1.0)  # what unused slots hold must not matter
+    kc, vc = new_caches(total, hkv, D, page, dtype, DEV, fill=None if math.isnan(fill) else fill)
+    if math.isnan(fill):                                            # what unused slots hold must not matter
+        kc.fill_(fill), vc.fill_(fill)
     vt = vc.shape[4]
     width = max(pages_per)
     tables = torch.full((S, width), -1, dtype=torch.int32)
@@ -544,6 +546,35 @@ def test_paged_attention(hip, ref, dtype, hq, hkv, D, page, lens, q_lens, window
             _close(hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window), twin, dtype, "general")
         finally:
             hip[dtype].mfma_attention = True
+
+
+@pytest.mark.parametrize("sets", [1, 2])
+@pytest.mark.parametrize("hq,hkv,D,page,lens,q_lens,window", [
+    (8, 2, 128, 256, [700, 1300], [700, 900], None),               # pages of whole tiles: the run of whole tiles
+    (8, 2, 128, 64, [1100, 130], [300, 130], None),                # a portion after a prefix, a page a tile
+    (4, 1, 64, 128, [900], [900], 200),                            # a window: tiles cut at both ends
+    (6, 2, 96, 24, [333, 80], [333, 1], None),                     # pages that hold no whole tile
+    (3, 3, 32, 8, [150], [150], 70),
+    (2, 1, 256, 64, [400], [250], None),                           # one wave per SIMD: always one set
+    (5, 1, 160, 32, [130, 70], [130, 70], None),                   # five heads: a second chunk with one wave at work
+])
+def test_prefill_attention_with_one_and_two_sets_of_waves(hip, sets, hq, hkv, D, page, lens, q_lens, window):
+    """The matrix-core prefill kernel with its waves as one set and as two (the launcher's own choice
+    goes by the number of workgroups), against the plain whole-sequence attention; what the cache
+    holds where no key was written is not a number."""
+    from nano_vllm_amd.kernels import library
+    dtype = torch.bfloat16
+    q, kc, vc, batch, parts = _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed=11, fill=float("nan"))
+    scale = D ** -0.5
+    want = _plain_attention(*parts, lens, q_lens, scale, window).to(DEV)
+    lib = library.load("attn_prefill", "bf16")
+    lib.nva_attn_prefill_sets(sets)
+    try:
+        got = hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window)
+    finally:
+        lib.nva_attn_prefill_sets(-1)
+    _close(got, want.to(dtype), dtype, f"{sets} sets")
+    hip[dtype].check_faults()
 
 
 @pytest.mark.parametrize("seed", range(12))
