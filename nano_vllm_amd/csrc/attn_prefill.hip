@@ -70,11 +70,11 @@ struct Swizzle {
 // depend, and waits for all of them before it.  These are waited for by count (wait_loads_but) and
 // shown to the other waves by a barrier, as the schedule below says.
 __device__ __forceinline__ void load_to_lds(const __bf16* src, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory", "m0");
 }
 // the same from base (the same for the whole wave) + offset (bytes, per lane)
 __device__ __forceinline__ void load_to_lds(const __bf16* base, uint32_t offset, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offset), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory");
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(offset), "s"(base), "s"(__builtin_amdgcn_readfirstlane(lds)) : "memory", "m0");
 }
 
 template <int N>
