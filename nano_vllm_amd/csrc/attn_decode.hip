@@ -265,7 +265,8 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
     f32x4 acc[DT];
 #pragma unroll
     for (int i = 0; i < DT; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;      // the maximum in units of raw scores
+    const float c_exp = scale * 1.4426950408889634f;      // scale * log2(e)
     // The loads of the chunk after are issued, unconditionally and on one path, before the products
     // of the current chunk, so that a wave always has a chunk (16 KiB at head_dim 128) in flight and
     // the wait before the products covers exactly the current chunk's loads.
@@ -301,30 +302,33 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
             sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], qf[c], sa, 0, 0, 0);
             sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[c], qf[c], sb, 0, 0, 0);
         }
-        // this lane: head `col`, keys base + 8g + i (tile a) and base + 8g + 4 + i (tile b)
+        // this lane: head `col`, keys base + 8g + i (tile a) and base + 8g + 4 + i (tile b).  The
+        // maximum is taken of the raw scores (scale > 0) and the scale folded, with log2(e), into the
+        // exponent: p = 2^((s - m) * scale * log2 e), one fused multiply-add per score; the four lanes
+        // of a head exchange their maxima and sums without LDS.
         float s[8];
         float m_new = m_run;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int key = base + 8 * g + i;
-            const float v = (i < 4 ? sa[i] : sb[i - 4]) * scale;
-            s[i] = (key >= first && key < kv_len) ? v : -INFINITY;
+            s[i] = (key >= first && key < kv_len) ? (i < 4 ? sa[i] : sb[i - 4]) : -INFINITY;
             m_new = fmaxf(m_new, s[i]);
         }
-        m_new = fmaxf(m_new, __shfl_xor(m_new, 16, NVA_WAVE));
-        m_new = fmaxf(m_new, __shfl_xor(m_new, 32, NVA_WAVE));
+        m_new = nva_max_over_rows(m_new);
+        // a head that has seen no key yet keeps -inf as its maximum; exponents then use a finite
+        // stand-in so that -inf - (-inf) never arises
+        const float m_use = fmaxf(m_new, -1e30f);
+        const float neg_mc = -m_use * c_exp;
         float psum = 0.f;
         bf16x8 pf;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            const float p = (s[i] == -INFINITY) ? 0.f : __expf(s[i] - m_new);
-            const __bf16 pb16 = (__bf16)p;
+            const __bf16 pb16 = (__bf16)__builtin_amdgcn_exp2f(fmaf(s[i], c_exp, neg_mc));
             pf[i] = pb16;
             psum += (float)pb16;           // the sum of what the product below really uses
         }
-        psum += __shfl_xor(psum, 16, NVA_WAVE);
-        psum += __shfl_xor(psum, 32, NVA_WAVE);
-        const float alpha = (m_run == -INFINITY) ? 0.f : __expf(m_run - m_new);
+        psum = nva_sum_over_rows(psum);
+        const float alpha = __builtin_amdgcn_exp2f((fmaxf(m_run, -1e30f) - m_use) * c_exp);
         l_run = l_run * alpha + psum;
         m_run = m_new;
         // ---- O^T += V^T P^T
@@ -353,7 +357,7 @@ attn_decode_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __res
             for (int dt = 0; dt < DT; ++dt)
                 *reinterpret_cast<f32x4*>(po + 16 * dt + 4 * g) = acc[dt];
             if (g == 0) {
-                part_ml[slot * 2] = m_run;
+                part_ml[slot * 2] = m_run * scale;             // as the merge takes it: of the scaled scores
                 part_ml[slot * 2 + 1] = l_run;
             }
         }

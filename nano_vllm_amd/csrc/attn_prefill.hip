@@ -86,16 +86,6 @@ __device__ __forceinline__ void wait_loads_but() {          // until at most N l
 // wait for every load on its way to LDS.)
 __device__ __forceinline__ void barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// What the lanes 0..31 and the lanes 32..63 hold of x, each in all lanes of its half's number: one
-// vector instruction that swaps the upper half of one register with the lower half of another
-// (a shuffle would go through LDS and wait for it).
-__device__ __forceinline__ void both_halves(float x, float& lower, float& upper) {
-    unsigned a = __builtin_bit_cast(unsigned, x), b = a;
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-    lower = __builtin_bit_cast(float, a);
-    upper = __builtin_bit_cast(float, b);
-}
-
 template <int D, int SETS>
 __global__ void __launch_bounds__(SETS * PF_WAVES * NVA_WAVE, PF_WAVES_PER_SIMD(D))
 attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __restrict__ out, int64_t out_stride,
@@ -313,7 +303,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
 #pragma unroll
             for (int e = 0; e < 16; ++e) m_new = fmaxf(m_new, s[kt][e]);
         float of_lower, of_upper;
-        both_halves(m_new, of_lower, of_upper);
+        nva_lane_halves(m_new, of_lower, of_upper);
         m_new = fmaxf(of_lower, of_upper);
         // a row that has seen no key yet keeps -inf as its maximum; exponents then use a finite
         // stand-in so that -inf - (-inf) never arises
@@ -333,7 +323,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                 pf[kt][e >> 3][(e & 7) + 1] = pair[1];
                 psum = __builtin_amdgcn_fdot2_f32_bf16(pair, ones, psum, false);
             }
-        both_halves(psum, of_lower, of_upper);
+        nva_lane_halves(psum, of_lower, of_upper);
         psum = of_lower + of_upper;
         // The accumulators are rescaled only when some row of the wave has a new maximum (after the
         // first tiles of a row that is rare): alpha is exactly 1 otherwise.

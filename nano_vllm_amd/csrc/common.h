@@ -174,6 +174,36 @@ __device__ __forceinline__ void partial_value8(const PartialInput& p, int64_t ro
 }
 
 
+// Exchanges between the rows of 16 lanes of a wave by one vector instruction each (a shuffle goes
+// through LDS and waits for it).  nva_lane_halves: what the lanes 0..31 and the lanes 32..63 hold of
+// x, each in all lanes of its own lane number modulo 32.  nva_lane_rows: of each pair of rows (0 and
+// 1, 2 and 3) what the even and what the odd row holds, in both rows of the pair.
+__device__ __forceinline__ void nva_lane_halves(float x, float& lower, float& upper) {
+    unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    lower = __builtin_bit_cast(float, a);
+    upper = __builtin_bit_cast(float, b);
+}
+__device__ __forceinline__ void nva_lane_rows(float x, float& even, float& odd) {
+    unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    even = __builtin_bit_cast(float, a);
+    odd = __builtin_bit_cast(float, b);
+}
+// the maximum and the sum over the four lanes l, l + 16, l + 32, l + 48, in all four
+__device__ __forceinline__ float nva_max_over_rows(float x) {
+    float a, b;
+    nva_lane_rows(x, a, b);
+    nva_lane_halves(fmaxf(a, b), a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float nva_sum_over_rows(float x) {
+    float a, b;
+    nva_lane_rows(x, a, b);
+    nva_lane_halves(a + b, a, b);
+    return a + b;
+}
+
 // ---------------------------------------------------------------------------- cache layout
 // K [pages, kv_heads, page_size, head_dim].
 // V [pages, kv_heads, page_size / vt, head_dim, vt]: transposed (the keys of one channel are
