@@ -92,7 +92,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
                     const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                     const int32_t* __restrict__ block_tables, int table_stride,
                     const int32_t* __restrict__ cu_seqlens_q, const int32_t* __restrict__ kv_lens,
-                    const int32_t* __restrict__ tiles, int num_tiles, int num_q_heads, int num_kv_heads,
+                    const int32_t* __restrict__ tiles, int num_tiles, int paired, int num_q_heads, int num_kv_heads,
                     int page_size, float scale, int window, int32_t* error_flag) {
     constexpr int DC = D / 16;            // 16-channel steps of the first product
     constexpr int MT = D / 32;            // 32-channel tiles of the output
@@ -111,10 +111,18 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     // ---- which request, which 32 rows of it, which heads.  `tiles` lists (request, row tile) from the
     // most keys to the fewest; a rank counts (tile, head chunk) pairs in that order.  Workgroups are
     // handed out in the order of their index, to the XCDs in turn and within an XCD to its CUs in turn,
-    // one to a CU at a time: the heaviest go first and the light ones fill the gaps.  With as many
-    // head chunks as XCDs, a kv head's keys and values stay in one XCD's L2.
+    // as many to a CU as it holds: the heaviest go first and the light ones fill the gaps.  Where all
+    // of a step's workgroups are on the GPU at once, two to a CU (`paired`: their number then), the
+    // first half of the indices takes the heavy ranks in order and the second half the light ranks from
+    // the lightest, so that a CU's two workgroups are a heavy and a light one: the heavy one then works
+    // alone (at one wave per SIMD) for the shortest time the pairing allows.  With as many head chunks
+    // as XCDs, a kv head's keys and values stay in one XCD's L2.
     const int ny = num_kv_heads * ((num_q_heads / num_kv_heads + PF_WAVES - 1) / PF_WAVES);
-    const int rank = blockIdx.x;
+    int rank = blockIdx.x;
+    if (paired) {
+        const int heavy = 8 * ((paired + 15) / 16);
+        if (rank >= heavy) rank = paired - 1 - (rank - heavy);
+    }
     const int by = rank % ny;
     const int seq = tiles[2 * (rank / ny)], tile = tiles[2 * (rank / ny) + 1];
     const int q_begin = cu_seqlens_q[seq];
@@ -538,12 +546,14 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
         }
     }
     // two sets of waves in a workgroup where every CU gets one workgroup at most
-    const bool two_sets = forced_sets > 0 ? forced_sets == 2 : num_tiles * grid_y <= cus;
+    const int64_t total = num_tiles * grid_y;
+    const bool two_sets = forced_sets > 0 ? forced_sets == 2 : total <= cus;
 #define LAUNCH_SETS(DD, SS)                                                                                        \
     hipLaunchKernelGGL((attn_prefill_kernel<DD, SS>), grid, dim3(SS * PF_WAVES * NVA_WAVE), table_bytes, stream,     \
                        (const __bf16*)q, q_stride, (__bf16*)out, out_stride, (const __bf16*)k_cache,                 \
                        (const __bf16*)v_cache, block_tables, table_stride, cu_seqlens_q, kv_lens, tiles,             \
-                       (int)num_tiles, num_q_heads, num_kv_heads, page_size, scale, window, error_flag)
+                       (int)num_tiles, SS == 1 && PF_WAVES_PER_SIMD(DD) == 2 && total <= 2 * cus ? (int)total : 0,   \
+                       num_q_heads, num_kv_heads, page_size, scale, window, error_flag)
 #define LAUNCH(DD)                                                                                                 \
     do {                                                                                                           \
         if (PF_WAVES_PER_SIMD(DD) == 2 && two_sets) LAUNCH_SETS(DD, PF_WAVES_PER_SIMD(DD));                         \
