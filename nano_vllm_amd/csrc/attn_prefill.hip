@@ -203,9 +203,11 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
 
     // ---- the tiles' loads.  Load i of a wave fills the 64 slots from (4 i + wave) * 64 of the tile: of
     // K, slot n is row n / KR (a key), place n % KR; of V, row n / 8 (a channel), place n % 8 (eight
-    // keys).  Every load is unconditional: a key outside the visible range is replaced by the nearest
-    // visible one (its scores are masked by the key index; what V holds for it is cleared in LDS, in
-    // the tiles at the two ends only).
+    // keys).  Every load is unconditional.  Where pages hold whole tiles (page_size % 64 == 0) a tile's
+    // loads are one base address, held in scalar registers, plus an offset per lane that never changes;
+    // else every lane looks its key's page up, and a key outside the visible range is replaced by the
+    // nearest visible one.  Either way the scores of keys outside the range are masked by the key index
+    // and what V holds for them is cleared in LDS, in the tiles at the two ends only.
     //
     // The tiles fall into three runs: those the window's start cuts, those every row sees whole, and
     // those the diagonal cuts.  The middle run, most of a long prompt, runs without any masking, and
@@ -240,6 +242,14 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         const __bf16* base = (const __bf16*)((uint64_t)high << 32 | low);
 #pragma unroll
         for (int i = 0; i < PIECES; ++i) load_to_lds(base, off[i], lds + i * LOAD_BYTES);
+    };
+    // A tile in pages of whole tiles, wherever it lies: keys of it outside the visible range are
+    // fetched as they are (they lie in the tile's own page; the scores of such keys are masked by the
+    // key index and what V holds for them is cleared in LDS); a tile past the last is the last again.
+    auto load_in_page = [&](const __bf16* cache, int kb, const uint32_t* off, uint32_t lds) __attribute__((always_inline)) {
+        kb = min(kb, after_last);
+        const int page = __builtin_amdgcn_readfirstlane(table_s[kb / page_size - page_lo]);
+        load_fast(cache, page, kb % page_size, off, lds);
     };
     auto load_k_any = [&](int kb, int buf) __attribute__((always_inline)) {
         kb = min(kb, after_last);
@@ -412,10 +422,18 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
         barrier();
         buf ^= 1;
     };
+    auto load_k = [&](int kb, int b) __attribute__((always_inline)) {
+        if (fast_pages) load_in_page(k_cache, kb, k_off, lds_wave + b * 2 * TILE);
+        else load_k_any(kb, b);
+    };
+    auto load_v = [&](int kb, int b) __attribute__((always_inline)) {
+        if (fast_pages) load_in_page(v_cache, kb, v_off, lds_wave + (2 + b) * 2 * TILE);
+        else load_v_any(kb, b);
+    };
     auto round = [&](int kb, auto masked_tag) __attribute__((always_inline)) {
         if (active) softmax(kb, masked_tag);
-        load_k_any(kb + 2 * STEP, buf);
-        load_v_any(kb + STEP, buf ^ 1);
+        load_k(kb + 2 * STEP, buf);
+        load_v(kb + STEP, buf ^ 1);
         wait_loads_but<2 * PIECES>();
         if (decltype(masked_tag)::value && (kb < first_any || kb + PF_BN > kb_hi)) clear_v_outside(kb, buf);
         products();
@@ -446,9 +464,9 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     const int rounds = ((kb_hi - kb_lo + PF_BN - 1) / PF_BN + SETS - 1) / SETS;
     if (SETS > 1 && set == 1) barrier();
     int kb = kb_lo + set * PF_BN;
-    load_k_any(kb, 0);
-    load_k_any(kb + STEP, 1);
-    load_v_any(kb, 0);
+    load_k(kb, 0);
+    load_k(kb + STEP, 1);
+    load_v(kb, 0);
     wait_loads_but<2 * PIECES>();
     barrier();
     if (active) products_of(0, 0, No());
