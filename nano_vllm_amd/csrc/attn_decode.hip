@@ -41,10 +41,18 @@ __device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf1
     const int key_b = min(max(base + row_key + 4, first), kv_len - 1);
     // the group of 8 keys of V, moved to the nearest group that holds a visible key
     const int key0 = min(max(base + 8 * g, first & ~7), (kv_len - 1) & ~7);
-    // block table entries come from the wave's register window (lane i holds page window_page0 + i)
-    const int page_a = __shfl(table_window, (key_a / page_size - window_page0) & (NVA_WAVE - 1), NVA_WAVE);
-    const int page_b = __shfl(table_window, (key_b / page_size - window_page0) & (NVA_WAVE - 1), NVA_WAVE);
-    const int page_v = __shfl(table_window, (key0 / page_size - window_page0) & (NVA_WAVE - 1), NVA_WAVE);
+    // block table entries come from the wave's register window (lane i holds page window_page0 + i);
+    // a chunk begins at a multiple of its 32 keys, so where pages hold whole chunks it lies in one
+    // page, which one instruction reads from the window (a shuffle per key goes through LDS)
+    int page_a, page_b, page_v;
+    if (page_size % DEC_CHUNK == 0) {
+        page_a = page_b = page_v = __builtin_amdgcn_readlane(
+            table_window, __builtin_amdgcn_readfirstlane(base / page_size - window_page0) & (NVA_WAVE - 1));
+    } else {
+        page_a = __shfl(table_window, (key_a / page_size - window_page0) & (NVA_WAVE - 1), NVA_WAVE);
+        page_b = __shfl(table_window, (key_b / page_size - window_page0) & (NVA_WAVE - 1), NVA_WAVE);
+        page_v = __shfl(table_window, (key0 / page_size - window_page0) & (NVA_WAVE - 1), NVA_WAVE);
+    }
     if (page_a < 0 || page_b < 0 || page_v < 0) {
         if (error_flag) atomicOr(error_flag, 2);
     }
