@@ -577,6 +577,29 @@ def test_prefill_attention_with_one_and_two_sets_of_waves(hip, sets, hq, hkv, D,
     hip[dtype].check_faults()
 
 
+@pytest.mark.parametrize("page", [64, 256, 24])
+def test_prefill_attention_behind_a_window_whose_first_pages_were_given_back(hip, page):
+    """A portion late in a long request behind a window: the block table has no page (-1) where no
+    row sees a key any more, the kernel reads page 0 for such entries, and page 0 holds no numbers."""
+    dtype, hq, hkv, D, window = torch.bfloat16, 4, 2, 128, 300
+    lens, q_lens = [1500], [200]
+    q, kc, vc, batch, parts = _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed=17, fill=float("nan"))
+    tables = batch.groups[0].block_tables
+    # page 0 is made free: what it holds moves to a page nobody uses, which the table then names
+    used = set(tables.flatten().tolist())
+    spare = next(i for i in range(kc.shape[0]) if i not in used and i != 0)
+    kc[spare], vc[spare] = kc[0], vc[0]
+    tables[tables == 0] = spare
+    kc[0], vc[0] = float("nan"), float("nan")
+    first_seen = lens[0] - q_lens[0] - window + 1                  # the first key the portion's first row sees
+    tables[0, : first_seen // page] = -1
+    scale = D ** -0.5
+    want = _plain_attention(*parts, lens, q_lens, scale, window).to(DEV)
+    got = hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window)
+    _close(got, want.to(dtype), dtype, f"page {page}")
+    hip[dtype].check_faults()
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_attention_of_drawn_shapes(hip, ref, seed):
     """Head counts, groups, head sizes, page sizes, windows and lengths drawn at random (single tokens
