@@ -66,6 +66,12 @@ def cmd_throughput(args) -> int:
     import random
     import time
     from . import LLM, SamplingParams
+    for what, low, high in (("input", args.min_input_len, args.max_input_len),
+                            ("output", args.min_output_len, args.max_output_len)):
+        if not 1 <= low <= high:
+            print(f"throughput: --min-{what}-len {low} and --max-{what}-len {high} must satisfy 1 <= min <= max",
+                  file=sys.stderr)
+            return 2
     rng = random.Random(args.workload_seed)
     llm = LLM(args.model, **engine_kwargs(args))
     vocab = llm.model.spec.vocab_size

@@ -23,3 +23,9 @@ def test_random_model_command_writes_a_shape(tmp_path, capsys):
     assert main(["random-model", "--shape", "tiny-b", "--seed", "2", "--out", str(tmp_path / "m")]) == 0
     assert (tmp_path / "m" / "model.safetensors").exists()
     assert main(["random-model", "--out", str(tmp_path / "x")]) == 2
+
+
+def test_throughput_command_refuses_an_empty_range_of_lengths(capsys):
+    assert main(["throughput", "--model", "nowhere", "--max-output-len", "64"]) == 2       # the minimum's default is 100
+    assert "--min-output-len 100 and --max-output-len 64" in capsys.readouterr().err
+    assert main(["throughput", "--model", "nowhere", "--min-input-len", "0"]) == 2
