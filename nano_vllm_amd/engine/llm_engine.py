@@ -125,10 +125,11 @@ class LLMEngine:
         seqs, is_prefill = self.scheduler.schedule()
         num_tokens = 0
         if seqs:
-            entries, sampled = [], []
+            entries, sampled, decoding = [], [], []
             for seq in seqs:
                 start, n = seq.num_cached_tokens, seq.num_scheduled_tokens
                 last = start + n == seq.num_tokens
+                decoding.append(n == 1 and last and seq.num_completion_tokens > 0)
                 entries.append(StepEntry(seq.seq_id, seq.token_ids[start:start + n], start, [n - 1] if last else []))
                 if last:
                     sampled.append(seq)
@@ -158,9 +159,10 @@ class LLMEngine:
                 self.scheduler.postprocess(seqs, [tokens.get(s.seq_id, -1) for s in seqs])
             num_tokens = sum(len(e.tokens) for e in entries) if is_prefill else -len(seqs)
             dt = perf_counter() - t0
-            kind = "prefill" if is_prefill else "decode"
-            self.stats[f"{kind}_tokens"] += abs(num_tokens)
-            self.stats[f"{kind}_time"] += dt
+            # tokens by what they are (a mixed step holds both kinds), time by the kind of the step
+            self.stats["prefill_tokens"] += sum(len(e.tokens) for e, d in zip(entries, decoding) if not d)
+            self.stats["decode_tokens"] += sum(decoding)
+            self.stats["prefill_time" if is_prefill else "decode_time"] += dt
             self.stats["steps"] += 1
         finished = self.scheduler.just_finished
         self.scheduler.just_finished = []

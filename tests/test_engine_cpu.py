@@ -140,6 +140,16 @@ def test_schedules_prefix_cache_and_page_shortage_do_not_change_the_tokens():
             assert llm.scheduler.num_preemptions > 0
 
 
+def test_the_engines_counts_tell_prompt_tokens_from_decoded_ones_in_either_schedule():
+    prompts = _prompts("a", (3, 9, 24, 40))
+    for kw in (dict(), dict(schedule="mixed"), dict(schedule="mixed", decode_burst=1)):
+        llm = _llm("a", enable_prefix_caching=False, **kw)
+        llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=7, ignore_eos=True), use_tqdm=False)
+        # a request's first token comes out of the step that holds the end of its prompt
+        assert llm.stats["prefill_tokens"] == sum(len(p) for p in prompts), kw
+        assert llm.stats["decode_tokens"] == len(prompts) * 6, kw
+
+
 def test_temperature_sampling_is_the_plain_draw_and_is_reproducible():
     prompts = _prompts("a", (5, 11))
     sp = SamplingParams(temperature=0.7, max_tokens=5, seed=42)
