@@ -8,7 +8,7 @@ or a head with a cap on its logits is another kind, registered): Model knows no 
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Mapping, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import torch
 
