@@ -4,82 +4,135 @@
 //
 // This is the tiled kernel on the vector units: inputs are read as they are stored, every
 // product and sum is a float operation (no matrix-core instruction, no reduced-precision
-// input format), and each output is summed over k in ascending order in 16-wide tiles,
-// whatever M is.  It is the matrix product of the 32-bit path and accepts any M, N, K.
-// The result is written as elements or, for logits, as float.
+// input format), and each output is one chain of multiply-adds over k in ascending order,
+// whatever M is and whichever tile shape runs: the result does not depend on the batch.  It is the
+// matrix product of the 32-bit path and accepts any M, N, K.  The result is written as elements
+// or, for logits, as float.
+//
+// A workgroup of 256 threads takes BM rows of x and BN rows of W; a thread TM x TN outputs, in
+// groups of up to four consecutive rows and columns BM / GM and BN / GN apart (the reads of LDS are
+// then 16 bytes per lane, neighbours side by side).  The tiles of x and W go through LDS k-major,
+// BK columns at a time, in two buffers: the next tile's global loads are on their way while this
+// one is multiplied, one barrier per tile.  Four shapes: 128 x 128 where that gives every CU a
+// workgroup, else 64 x 64; for the few rows of a decode step, where W is streamed once, 16 x 64 with
+// tiles of 64 columns (four rows a thread: its reads of x are one broadcast), or 16 x 16 where W has too
+// few rows to give every CU a workgroup of 64 of them.
 #include "common.h"
 
-#define TILE_M 64
-#define TILE_N 64
-#define TILE_K 16
-
 template <typename T>
-__device__ __forceinline__ void load_tile(const T* __restrict__ src, int64_t stride, int rows_left, int k_left,
-                                          bool vec, float (*dst)[TILE_M + 4], int tid) {
-    // 64 rows x 16 k: each of the 256 threads takes 4 consecutive k of one row
-    const int r = tid / 4, kq = (tid % 4) * 4;
-    float v[4] = {0.f, 0.f, 0.f, 0.f};
-    if (r < rows_left) {
-        const T* p = src + (int64_t)r * stride + kq;
-        if (vec && kq + 4 <= k_left) {
-            if (sizeof(T) == 4) {
-                const float4 f = *reinterpret_cast<const float4*>(p);
-                v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
-            } else {
-                typedef __attribute__((ext_vector_type(4))) __bf16 b4;
-                const b4 f = *reinterpret_cast<const b4*>(p);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = static_cast<float>(f[e]);
-            }
+__device__ __forceinline__ void load4(const T* __restrict__ p, bool whole, int k_left, float v[4]) {
+    if (whole) {
+        if (sizeof(T) == 4) {
+            const float4 f = *reinterpret_cast<const float4*>(p);
+            v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
         } else {
+            typedef __attribute__((ext_vector_type(4))) __bf16 b4;
+            const b4 f = *reinterpret_cast<const b4*>(p);
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (kq + e < k_left) v[e] = to_float(p[e]);
+            for (int e = 0; e < 4; ++e) v[e] = static_cast<float>(f[e]);
         }
-    }
+    } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) dst[kq + e][r] = v[e];
+        for (int e = 0; e < 4; ++e) v[e] = e < k_left ? to_float(p[e]) : 0.f;
+    }
 }
 
-template <typename T, typename OutT>
-__global__ void __launch_bounds__(256)
+// R rows x BK columns of a matrix, from its row `row0` and column k0, as 4-column pieces: piece p of
+// a thread is number tid + 256 p; its row is number / (BK / 4).  Rows and columns past the end are zeros.
+template <typename T, int R, int BK>
+struct TileLoad {
+    static constexpr int PIECES = R * BK / 4 / 256;
+    static_assert(R * BK / 4 % 256 == 0 && PIECES >= 1, "a tile is a whole number of pieces per thread");
+    float v[PIECES][4];
+    __device__ __forceinline__ void fetch(const T* __restrict__ src, int64_t stride, int rows_left, int k_left, bool vec, int tid) {
+#pragma unroll
+        for (int p = 0; p < PIECES; ++p) {
+            const int n = tid + 256 * p, r = n / (BK / 4), kq = (n % (BK / 4)) * 4;
+            if (r < rows_left && kq < k_left) {
+                load4<T>(src + (int64_t)r * stride + kq, vec && kq + 4 <= k_left, k_left - kq, v[p]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[p][e] = 0.f;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(float (*dst)[R + 4], int tid) const {
+#pragma unroll
+        for (int p = 0; p < PIECES; ++p) {
+            const int n = tid + 256 * p, r = n / (BK / 4), kq = (n % (BK / 4)) * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dst[kq + e][r] = v[p][e];
+        }
+    }
+};
+
+template <typename T, typename OutT, int BM, int BN, int BK, int TM, int TN>
+__global__ void __launch_bounds__(256, 2)
 linear_tiled_kernel(const T* __restrict__ x, int64_t x_stride, const T* __restrict__ w, int64_t w_stride,
                     const T* __restrict__ bias, OutT* __restrict__ y, int64_t y_stride, int M, int N, int K,
                     int vec) {
-    __shared__ float xs[TILE_K][TILE_M + 4];
-    __shared__ float ws[TILE_K][TILE_N + 4];
+    constexpr int VM = TM >= 4 ? 4 : TM, GM = TM / VM;       // a thread's rows: GM groups of VM consecutive ones
+    constexpr int VN = TN >= 4 ? 4 : TN, GN = TN / VN;
+    constexpr int TX = BN / TN;                               // threads side by side along n
+    static_assert((BM / TM) * TX == 256, "256 threads cover the tile");
+    __shared__ float xs[2][BK][BM + 4];
+    __shared__ float ws[2][BK][BN + 4];
     const int tid = threadIdx.x;
-    const int m0 = blockIdx.y * TILE_M, n0 = blockIdx.x * TILE_N;
-    const int ty = tid / 16, tx = tid % 16;
-    float acc[4][4];
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const int ty = tid / TX, tx = tid % TX;
+    float acc[TM][TN];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+        for (int j = 0; j < TN; ++j) acc[i][j] = 0.f;
 
-    for (int k0 = 0; k0 < K; k0 += TILE_K) {
-        load_tile<T>(x + (int64_t)m0 * x_stride + k0, x_stride, M - m0, K - k0, vec, xs, tid);
-        load_tile<T>(w + (int64_t)n0 * w_stride + k0, w_stride, N - n0, K - k0, vec, ws, tid);
-        __syncthreads();
+    TileLoad<T, BM, BK> lx;
+    TileLoad<T, BN, BK> lw;
+    const T* xp = x + (int64_t)m0 * x_stride;
+    const T* wp = w + (int64_t)n0 * w_stride;
+    lx.fetch(xp, x_stride, M - m0, K, vec, tid);
+    lw.fetch(wp, w_stride, N - n0, K, vec, tid);
+    lx.store(xs[0], tid);
+    lw.store(ws[0], tid);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        const bool more = k0 + BK < K;
+        if (more) {
+            lx.fetch(xp + k0 + BK, x_stride, M - m0, K - k0 - BK, vec, tid);
+            lw.fetch(wp + k0 + BK, w_stride, N - n0, K - k0 - BK, vec, tid);
+        }
+#pragma unroll 4
+        for (int k = 0; k < BK; ++k) {
+            float av[TM], bv[TN];
 #pragma unroll
-        for (int k = 0; k < TILE_K; ++k) {
-            const float4 a = *reinterpret_cast<const float4*>(&xs[k][ty * 4]);
-            const float4 b = *reinterpret_cast<const float4*>(&ws[k][tx * 4]);
-            const float av[4] = {a.x, a.y, a.z, a.w}, bv[4] = {b.x, b.y, b.z, b.w};
+            for (int g = 0; g < GM; ++g)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < VM; ++i) av[g * VM + i] = xs[buf][k][g * (BM / GM) + ty * VM + i];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] += av[i] * bv[j];
+            for (int g = 0; g < GN; ++g)
+#pragma unroll
+                for (int j = 0; j < VN; ++j) bv[g * VN + j] = ws[buf][k][g * (BN / GN) + tx * VN + j];
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) acc[i][j] += av[i] * bv[j];
+        }
+        if (more) {
+            // the other buffer was last read before the barrier that ended the previous tile
+            lx.store(xs[buf ^ 1], tid);
+            lw.store(ws[buf ^ 1], tid);
         }
         __syncthreads();
+        buf ^= 1;
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int m = m0 + ty * 4 + i;
+    for (int i = 0; i < TM; ++i) {
+        const int m = m0 + (i / VM) * (BM / GM) + ty * VM + i % VM;
         if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int n = n0 + tx * 4 + j;
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + (j / VN) * (BN / GN) + tx * VN + j % VN;
             if (n >= N) continue;
             float v = acc[i][j];
             if (bias) v += to_float(bias[n]);
@@ -94,19 +147,35 @@ NVA_EXPORT int NVA_NAME(nva_linear_tiled)(const void* x, int64_t x_stride, const
     if (M == 0 || N == 0) return 0;
     if (M < 0 || N < 0 || K <= 0 || M > 0x7fffffff || N > 0x7fffffff || K > 0x7fffffff)
         return nva_fail("linear: bad shape M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-    const int64_t grid_m = (M + TILE_M - 1) / TILE_M, grid_n = (N + TILE_N - 1) / TILE_N;
-    if (grid_m > 65535) return nva_fail("linear: M=%lld exceeds %d rows per call", (long long)M, 65535 * TILE_M);
     const size_t vb = 4 * sizeof(elem_t);
     const int vec = x_stride % 4 == 0 && w_stride % 4 == 0 && nva_aligned(x, vb) && nva_aligned(w, vb);
-    dim3 grid((unsigned)grid_n, (unsigned)grid_m);
-    if (out_is_f32)
-        hipLaunchKernelGGL((linear_tiled_kernel<elem_t, float>), grid, dim3(256), 0, stream, (const elem_t*)x, x_stride,
-                           (const elem_t*)w, w_stride, (const elem_t*)bias, (float*)y, y_stride, (int)M, (int)N,
-                           (int)K, vec);
-    else
-        hipLaunchKernelGGL((linear_tiled_kernel<elem_t, elem_t>), grid, dim3(256), 0, stream, (const elem_t*)x,
-                           x_stride, (const elem_t*)w, w_stride, (const elem_t*)bias, (elem_t*)y, y_stride, (int)M,
-                           (int)N, (int)K, vec);
+#define LAUNCH_AS(OUT, BM, BN, BK, TM, TN)                                                                            \
+    hipLaunchKernelGGL((linear_tiled_kernel<elem_t, OUT, BM, BN, BK, TM, TN>), grid, dim3(256), 0, stream,            \
+                       (const elem_t*)x, x_stride, (const elem_t*)w, w_stride, (const elem_t*)bias, (OUT*)y, y_stride, \
+                       (int)M, (int)N, (int)K, vec)
+#define LAUNCH(BM, BN, BK, TM, TN)                                                                                    \
+    do {                                                                                                              \
+        const int64_t grid_m = (M + BM - 1) / BM, grid_n = (N + BN - 1) / BN;                                         \
+        if (grid_m > 65535) return nva_fail("linear: M=%lld exceeds %d rows per call", (long long)M, 65535 * BM);     \
+        dim3 grid((unsigned)grid_n, (unsigned)grid_m);                                                                \
+        if (out_is_f32) LAUNCH_AS(float, BM, BN, BK, TM, TN);                                                         \
+        else LAUNCH_AS(elem_t, BM, BN, BK, TM, TN);                                                                   \
+    } while (0)
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+            cus = 0;
+            return nva_fail("linear: cannot read the number of CUs");
+        }
+    }
+    if (M <= 16) {
+        if (N >= 64 * (int64_t)cus) LAUNCH(16, 64, 64, 4, 1);
+        else LAUNCH(16, 16, 64, 1, 1);
+    } else if (((M + 127) / 128) * ((N + 127) / 128) >= cus) LAUNCH(128, 128, 16, 8, 8);
+    else LAUNCH(64, 64, 16, 4, 4);
+#undef LAUNCH
+#undef LAUNCH_AS
     return nva_check_launch("linear_tiled");
 }
 

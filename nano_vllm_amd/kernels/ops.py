@@ -100,6 +100,7 @@ def check_positions_fit(table: torch.Tensor, head_dim: int, max_position: Option
 MEDIUM_KERNEL_ROWS = 256    # rows of x that nva_linear_medium takes
 PREFILL_ROWS = 32       # query rows of one workgroup of the prefill attention kernel
 PREFILL_MAX_TABLE = 4096    # pages of a block-table row the prefill attention kernel stages in LDS
+GENERAL_TILED_MAX_HEAD_DIM = 128    # head sizes of nva_paged_attention_tiled
 
 
 def prefill_tile_order(q_lens, starts, first_seq: int) -> list:
@@ -153,6 +154,8 @@ class HipKernels:
         self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
         self.mfma_attention = True
+        # False: the general kernel runs one wave per token for portions of prompts too (the same bits, slower)
+        self.tiled_general_attention = True
 
     # ------------------------------------------------------------------ helpers
     def _stream(self):
@@ -661,29 +664,46 @@ class HipKernels:
         if start < tokens and q.dtype == torch.bfloat16 and self.mfma_attention and start == batch.num_decode and \
                 self._prefill_kernel_takes(head_dim, page_size, tables.shape[1], q, qs, out, os_):
             # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
-            tiles = getattr(batch, "prefill_tiles", None)
-            if tiles is None:       # a batch that was not built by the engine: order the tiles here, once
-                flat = prefill_tile_order(batch.q_lens, batch.starts if getattr(batch, "starts", None) else
-                                          [int(kv) - n for kv, n in zip(batch.kv_lens.tolist(), batch.q_lens)],
-                                          batch.num_decode)
-                tiles = torch.tensor(flat, dtype=torch.int32, device=q.device).view(-1, 2)
-                batch.prefill_tiles = tiles
-            if tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 2 or not tiles.is_contiguous():
-                raise KernelError("attention: prefill_tiles must be contiguous int32 [tiles, 2]")
+            tiles = self._prefill_tiles(batch, q.device)
             library.call("attn_prefill", "bf16", "nva_attn_prefill", _p(q), c_i64(qs), _p(out), c_i64(os_), _p(k_cache),
                          _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q), _p(batch.kv_lens),
                          _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
                          _p(self.fault_flag), self._stream())
             start = tokens
+        if self.tiled_general_attention and start <= batch.num_decode < tokens and not window and \
+                head_dim <= GENERAL_TILED_MAX_HEAD_DIM:
+            # portions of prompts in float arithmetic: the per-token kernel's arithmetic, operation for
+            # operation, with the keys staged once for 32 query rows
+            tiles = self._prefill_tiles(batch, q.device)
+            library.call("attn_generic", _suffix(q), "nva_paged_attention_tiled", _p(q), c_i64(qs), _p(out), c_i64(os_),
+                         _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]), _p(batch.cu_seqlens_q),
+                         _p(batch.kv_lens), _p(tiles), c_i64(tiles.shape[0]), c_i32(num_heads), c_i32(num_kv_heads),
+                         c_i32(head_dim), c_i32(page_size), c_f32(scale), _p(self.fault_flag), self._stream())
+            tokens = batch.num_decode            # what is left: the single tokens before the portions
         if start < tokens:
             n = tokens - start
-            library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q[start:]), c_i64(qs),
+            library.call("attn_generic", _suffix(q), "nva_paged_attention_generic", _p(q[start:start + n]), c_i64(qs),
                          _p(out[start:]), c_i64(os_), _p(k_cache), _p(v_cache), _p(tables), c_i32(tables.shape[1]),
                          _p(batch.token_seq[start:]), _p(batch.positions[start:]), c_i64(n), c_i32(num_heads),
                          c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), c_f32(scale), c_i32(window or 0),
                          _p(self.fault_flag), self._stream())
         return out
+
+    @staticmethod
+    def _prefill_tiles(batch, device) -> torch.Tensor:
+        """int32 [tiles, 2] = (request, tile of 32 query rows) of the step's portions of prompts, from the
+        most keys to the fewest; a batch that was not built by the engine gets them here, once."""
+        tiles = getattr(batch, "prefill_tiles", None)
+        if tiles is None:
+            flat = prefill_tile_order(batch.q_lens, batch.starts if getattr(batch, "starts", None) else
+                                      [int(kv) - n for kv, n in zip(batch.kv_lens.tolist(), batch.q_lens)],
+                                      batch.num_decode)
+            tiles = torch.tensor(flat, dtype=torch.int32, device=device).view(-1, 2)
+            batch.prefill_tiles = tiles
+        if tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 2 or not tiles.is_contiguous():
+            raise KernelError("attention: prefill_tiles must be contiguous int32 [tiles, 2]")
+        return tiles
 
     @staticmethod
     def _decode_kernel_takes(group, head_dim, page_size, q, q_stride, out, out_stride) -> bool:

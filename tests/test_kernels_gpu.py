@@ -120,6 +120,16 @@ def test_linear_float32_does_not_depend_on_the_rows_beside_it(hip):
     whole = k.linear(x, w)
     assert torch.equal(k.linear(x[17:18], w), whole[17:18])         # bit for bit: the order of the sum is fixed
     assert torch.equal(k.linear(x[:3], w), whole[:3])
+    # every tile shape of the kernel: many rows on a wide weight (128 x 128), fewer (64 x 64), up to 16
+    # rows on a weight of few rows (16 x 16) and on one of many (16 x 64)
+    x, w = _rand((2100, 77), torch.float32, 13), _rand((17000, 77), torch.float32, 14)
+    whole = k.linear(x, w)
+    want = x.double() @ w.double().T
+    assert float((whole.double() - want).abs().max()) <= 1e-5 * float(want.abs().max())
+    assert torch.equal(k.linear(x[1999:2049], w), whole[1999:2049])
+    assert torch.equal(k.linear(x[5:6], w), whole[5:6])
+    assert torch.equal(k.linear(x[40:56], w[:1000]), whole[40:56, :1000])
+    assert torch.equal(k.linear(x[:100], w[300:500]), whole[:100, 300:500])
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 1001, 96), (5, 384, 120), (70, 777, 256), (3, 64, 4096)])
@@ -546,6 +556,30 @@ def test_paged_attention(hip, ref, dtype, hq, hkv, D, page, lens, q_lens, window
             _close(hip[dtype].paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, window), twin, dtype, "general")
         finally:
             hip[dtype].mfma_attention = True
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,D,page,lens,q_lens", [case[:6] for case in ATT_CASES if case[6] is None and case[2] <= 128] + [
+    (4, 2, 128, 256, [700, 90, 300], [1, 90, 257], ),              # a single token, a whole prompt, a portion behind 43 keys
+    (3, 3, 40, 8, [77, 130], [33, 130]),                           # a head size that is no multiple of 8
+    (2, 1, 112, 24, [100], [64]),
+])
+def test_general_attention_of_portions_gives_the_bits_of_one_wave_per_token(hip, dtype, hq, hkv, D, page, lens, q_lens):
+    """The general kernel has a form for portions of prompts that stages the keys once for 32 rows; its
+    arithmetic is the per-token kernel's, so the results are equal bit for bit, unused cache slots
+    holding no numbers."""
+    q, kc, vc, batch, parts = _paged_case(dtype, hq, hkv, D, page, lens, q_lens, seed=13, fill=float("nan"))
+    k, scale = hip[dtype], D ** -0.5
+    k.mfma_attention = False
+    try:
+        tiled = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, None)
+        k.tiled_general_attention = False
+        per_token = k.paged_attention(q, hq, hkv, D, kc, vc, batch, 0, scale, None)
+    finally:
+        k.mfma_attention = k.tiled_general_attention = True
+    k.check_faults()
+    assert torch.equal(tiled, per_token)
+    _close(tiled, _plain_attention(*parts, lens, q_lens, scale, None).to(DEV).to(dtype), dtype)
 
 
 @pytest.mark.parametrize("sets", [1, 2])
