@@ -384,12 +384,12 @@ NVA_EXPORT int NVA_NAME(nva_paged_attention_tiled)(
         return nva_fail("paged_attention_tiled: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
     if (page_size <= 0 || table_stride <= 0) return nva_fail("paged_attention_tiled: bad page size or table width");
     const size_t lds = att_tiled_lds(head_dim);
-    static bool raised[2] = {false, false};
     auto kernel = paged_attention_tiled_kernel<elem_t>;
-    if (!raised[sizeof(elem_t) == 4]) {
+    static bool raised = false;              // the kernel's LDS limit, lifted once to what the largest head size needs
+    if (!raised) {
         if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)att_tiled_lds(ATT_TILED_MAX_D)) != hipSuccess)
             return nva_fail("paged_attention_tiled: cannot have %zu bytes of LDS", att_tiled_lds(ATT_TILED_MAX_D));
-        raised[sizeof(elem_t) == 4] = true;
+        raised = true;
     }
     dim3 grid((unsigned)num_tiles, (unsigned)num_q_heads);
     hipLaunchKernelGGL(kernel, grid, dim3(ATT_TILED_WAVES * NVA_WAVE), lds, stream, (const elem_t*)q, q_stride,
