@@ -56,6 +56,37 @@ def test_one_request(runners, name, dtype, driving):
     r.kernels.check_faults()
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Every size and option of the configuration drawn at random (head sizes in steps of 16, odd
+    numbers of heads and groups, widths and vocabularies that are no power of two, with and without
+    the bias on q/k/v and the tied head), a page size, a dtype and a length: whole, the last tokens
+    one by one, and in portions, against the plain implementation."""
+    import random
+    from nano_vllm_amd.models.qwen3 import Qwen3Config
+    from nano_vllm_amd.weights import write_random_model
+    rng = random.Random(9000 + seed)
+    hkv, group = rng.choice([1, 2, 3, 4]), rng.choice([1, 2, 3, 4, 8])
+    cfg = Qwen3Config(vocab_size=rng.randint(50, 1500), hidden_size=8 * rng.randint(4, 40), num_hidden_layers=rng.randint(1, 3),
+                      num_attention_heads=hkv * group, num_key_value_heads=hkv,
+                      head_dim=rng.choice([16, 32, 48, 64, 80, 96, 128]), intermediate_size=8 * rng.randint(4, 60),
+                      rms_norm_eps=rng.choice([1e-6, 1e-5, 3e-4]), rope_theta=rng.choice([1e4, 5e5, 1e6]),
+                      max_position_embeddings=512, tie_word_embeddings=rng.random() < 0.5,
+                      attention_bias=rng.random() < 0.25)
+    page = rng.choice([4, 8, 16, 24, 32, 64, 256])
+    dtype = rng.choice(["float32", "bfloat16"])
+    n = rng.randint(3, 300)
+    folder = str(tmp_path / "model")
+    write_random_model(folder, cfg, seed=seed, norm_std=0.1, dtype=dtype)
+    toks = H.random_tokens(cfg.vocab_size, n, 40 + seed)
+    want = H.plain_logits(folder, toks, ROUNDING[dtype])
+    r = H.make_runner(folder, dtype, page, (512 + page - 1) // page + 4)
+    for portions in (H.whole(n), H.last_one_by_one(n, rng.randint(1, 40)), H.changing_portions(n, seed)):
+        got = H.run_portions(r, "x", toks, portions)
+        r.kernels.check_faults()
+        assert H.rel_err(got, want) < TOL[dtype], (cfg, page, dtype, n, portions[:4])
+
+
 @pytest.mark.parametrize("name", ["b", "d"])
 def test_decoding_with_the_kernel_for_wide_weights_forced(name):
     """At the tiny sizes no weight is wide enough for the kernel whose waves split k inside a
