@@ -64,6 +64,44 @@ def test_schedules_and_page_shortage_do_not_change_greedy_tokens():
             assert llm.scheduler.num_preemptions > 0
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_scheduling_options_drawn_at_random_do_not_change_the_tokens(tmp_path, seed):
+    """A configuration, requests (some sharing a prefix) and sampling drawn at random; then schedule,
+    pool size (down to what the longest request needs and one page), token budget, request limit, burst
+    length and prefix reuse drawn at random: the tokens of a run with plenty of everything, in
+    float32, where the logits do not depend on the batch by a bit."""
+    import random
+    from nano_vllm_amd.models.qwen3 import Qwen3Config
+    from nano_vllm_amd.weights import write_random_model
+    rng = random.Random(7000 + seed)
+    hkv, group = rng.choice([1, 2, 4]), rng.choice([1, 2, 4, 8])
+    cfg = Qwen3Config(vocab_size=rng.randint(50, 1500), hidden_size=8 * rng.randint(4, 30), num_hidden_layers=rng.randint(1, 3),
+                      num_attention_heads=hkv * group, num_key_value_heads=hkv, head_dim=rng.choice([16, 32, 64, 128]),
+                      intermediate_size=8 * rng.randint(4, 40), rms_norm_eps=1e-6, rope_theta=1e6, max_position_embeddings=512,
+                      tie_word_embeddings=rng.random() < 0.5)
+    page = rng.choice([4, 8, 16, 32, 64])
+    folder = str(tmp_path / "model")
+    write_random_model(folder, cfg, seed=seed, norm_std=0.1, dtype="float32")
+    count = rng.randint(2, 7)
+    prompts = [H.random_tokens(cfg.vocab_size, rng.randint(1, 150), 50 * seed + i) for i in range(count)]
+    if count > 2:
+        prompts[1] = prompts[0][:len(prompts[0]) // 2] + prompts[1][:5]
+    params = [SamplingParams(temperature=rng.choice([0.0, 0.0, 0.8]), max_tokens=rng.randint(1, 40), seed=rng.randint(0, 5))
+              for _ in prompts]
+    pages = [(len(p) + sp.max_tokens + page - 1) // page for p, sp in zip(prompts, params)]
+    plenty = dict(dtype="float32", kvcache_block_size=page, num_kvcache_blocks=sum(pages) + 4, max_num_batched_tokens=4096,
+                  max_num_seqs=8, decode_burst=1, enable_prefix_caching=False, max_model_len=512)
+    base = [o["token_ids"] for o in LLM(folder, **plenty).generate(prompts, params, use_tqdm=False)]
+    for _ in range(2):
+        kw = dict(plenty, schedule=rng.choice(["prefill_first", "mixed"]),
+                  num_kvcache_blocks=rng.choice([sum(pages) + 4, max(pages) + 1, max(pages) + rng.randint(1, 6)]),
+                  max_num_batched_tokens=rng.choice([4096, 16, rng.randint(2, 64)]), max_num_seqs=rng.choice([8, 1, 2, 3]),
+                  decode_burst=rng.choice([1, 2, 4, 8, 16]), enable_prefix_caching=rng.random() < 0.5)
+        llm = LLM(folder, **kw)
+        assert [o["token_ids"] for o in llm.generate(prompts, params, use_tqdm=False)] == base, kw
+        llm.runner.cache.check()
+
+
 def test_temperature_sampling_is_reproducible_and_independent_of_the_batch():
     name = "b"
     prompts = [H.random_tokens(384, n, 400 + n) for n in (7, 19, 31)]
