@@ -9,7 +9,11 @@ a batch of 8 requests and a context of 4096 tokens: after W untimed steps, K dec
 (one token per request and step, through the engine's step function and sampler) are timed
 so that the last one ends at the context length.  The cache in front of the timed steps is
 filled with random keys and values (a decode step's work does not depend on their values).
-Also measured: a prefill of 2,048 tokens, and decoding at batch 1 and 64.
+Also measured: a prefill of 2,048 tokens, decoding at batch 1 and 64, decoding at the default
+batch with a context of 32,768 tokens, and ("serve_256") the reference's own benchmark workload
+(bench.py:8-28 there: 256 requests of random ids, prompts and outputs of 100 to 1024 tokens,
+temperature 0.6, ignore_eos, one `generate` call after a short warm-up request) through
+`LLM.generate`: scheduler, chunked prefill, sampling and the host's round trips included.
 
 One JSON line is printed: `value` is decoded tokens a second at the default batch.
 The reference measures throughput the same way on synthetic token ids (bench.py:8-28 there).
@@ -40,7 +44,45 @@ def parse_args():
     ap.add_argument("--burst", type=int, default=None,
                     help="decode steps in a row without the host in between (default: the engine's decode_burst; 1: one)")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--long-context", type=int, default=32768,
+                    help="context of one more decode point at the default batch (0: none)")
+    ap.add_argument("--serve-seqs", type=int, default=256,
+                    help="requests of the reference's benchmark workload through LLM.generate (0: not run)")
     return ap.parse_args()
+
+
+def serve_run(args, config_json):
+    """The reference's benchmark (bench.py:8-28 there) on this model shape with random weights:
+    generated tokens a second of one generate call, and the engine's own split of it."""
+    import json as _json
+    import os
+    import random
+    import tempfile
+    from nano_vllm_amd import LLM, SamplingParams
+    rng = random.Random(0)
+    n = args.serve_seqs
+    prompts = [[rng.randint(0, 10000) for _ in range(rng.randint(100, 1024))] for _ in range(n)]
+    params = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=rng.randint(100, 1024)) for _ in range(n)]
+    with tempfile.TemporaryDirectory() as folder:
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            _json.dump(config_json, f)
+        llm = LLM(folder, random_weights=args.seed, max_model_len=4096, kvcache_block_size=args.page_size,
+                  enforce_eager=args.eager, **({} if args.burst is None else {"decode_burst": max(1, args.burst)}))
+        llm.generate([[1, 2, 3, 4]], SamplingParams(temperature=0.6, max_tokens=8, ignore_eos=True), use_tqdm=False)
+        for k in llm.stats:
+            llm.stats[k] = 0 if isinstance(llm.stats[k], int) else 0.0
+        t0 = time.perf_counter()
+        llm.generate(prompts, params, use_tqdm=False)
+        dt = time.perf_counter() - t0
+        st = llm.stats
+    total = sum(p.max_tokens for p in params)
+    out = {"value": round(total / dt, 1), "unit": "generated tok/s", "seconds": round(dt, 2), "generated_tokens": total,
+           "prompt_tokens": sum(len(p) for p in prompts),
+           "prefill_tok_s": round(st["prefill_tokens"] / max(st["prefill_time"], 1e-9), 1),
+           "decode_tok_s": round(st["decode_tokens"] / max(st["decode_time"], 1e-9), 1), "steps": st["steps"]}
+    print(f"# serve {n} requests: {total} tokens in {dt:.2f} s = {total / dt:.0f} tok/s (prefill {out['prefill_tok_s']:.0f}, "
+          f"decode {out['decode_tok_s']:.0f} tok/s by the engine's own clock)", file=sys.stderr, flush=True)
+    return out
 
 
 def main():
@@ -95,9 +137,9 @@ def main():
     weight_bytes = (L * layer_params + H + V * H) * itemsize            # every weight a step uses, once
     kv_bytes_per_token = 2 * L * Hkv * D * itemsize
 
-    def decode_run(batch, steps, warmup):
+    def decode_run(batch, steps, warmup, runner=runner, context=args.context):
         """Timed decode steps that end with `context` tokens in each request's cache."""
-        start = args.context - (steps + warmup)
+        start = context - (steps + warmup)
         ids = [f"d{batch}-{i}" for i in range(batch)]
         for rid in ids:
             runner.cache.admit(rid)
@@ -130,11 +172,11 @@ def main():
         some_steps(steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        assert pos == args.context
+        assert pos == context
         for rid in ids:
             runner.cache.release(rid)
         # keys read per step: the mean context over the timed steps
-        mean_ctx = args.context - (steps - 1) / 2.0
+        mean_ctx = context - (steps - 1) / 2.0
         step_bytes = weight_bytes + batch * H * itemsize + batch * mean_ctx * kv_bytes_per_token
         return dt, step_bytes
 
@@ -168,13 +210,41 @@ def main():
     print(f"# prefill {T} tokens: {T / pre_s:.0f} tok/s, {pre_s * 1e3:.2f} ms", file=sys.stderr, flush=True)
     kernels.check_faults()
 
+    extra_points = {}
+    if args.long_context > args.context and args.dtype == "bfloat16":
+        # the default batch at a long context, on a runner of its own (its captured steps are sized
+        # for that length; the headline's runner stays as it was)
+        ctx = args.long_context
+        del runner
+        torch.cuda.empty_cache()
+        long_runner = ModelRunner(model, page, args.batch * ((ctx + page - 1) // page + 1), args.batch + 1,
+                                  enable_prefix_caching=False)
+        if not args.eager:
+            long_runner.enable_decode_graphs(args.batch, ctx + page)
+        for lc in long_runner.layer_caches:
+            lc.k.normal_(0, 1)
+            lc.v.normal_(0, 1)
+        steps = max(8, args.steps // 2)
+        dt, step_bytes = decode_run(args.batch, steps, args.warmup, runner=long_runner, context=ctx)
+        extra_points[f"decode_b{args.batch}_ctx{ctx}"] = round(args.batch * steps / dt, 2)
+        print(f"# decode batch {args.batch} at context {ctx}: {args.batch * steps / dt:.1f} tok/s, {dt / steps * 1e3:.3f} "
+              f"ms/step, {step_bytes / (dt / steps) / 1e9:.0f} GB/s", file=sys.stderr, flush=True)
+        kernels.check_faults()
+        del long_runner
+        runner = None
+    serve = None
+    if args.serve_seqs > 0 and args.dtype == "bfloat16":
+        serve = serve_run(args, config_json)
+        torch.cuda.synchronize()
+
     value, step_s, step_bytes = results[args.batch]
     achieved = step_bytes / step_s / 1e9
     shape_name = args.shape.replace("qwen", "Qwen").replace("b", "B") if args.shape.startswith("qwen3-") else args.shape
     short_dtype = "bf16" if args.dtype == "bfloat16" else "fp32"
     line = {
         "metric": f"decode tok/s @ batch {args.batch}, context {args.context}, {shape_name} shape {short_dtype} "
-                  f"(also batch {'/'.join(str(b) for b in points if b != args.batch) or '-'} and prefill tok/s @ {T} tok)",
+                  f"(also batch {'/'.join(str(b) for b in points if b != args.batch) or '-'} and prefill tok/s @ {T} tok"
+                  + (f"; serve_{args.serve_seqs}: the reference's bench.py workload through LLM.generate" if serve else "") + ")",
         "value": round(value, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": short_dtype, "data": "synthetic",
@@ -182,14 +252,16 @@ def main():
                    "parallelism": "single GPU", "layers": L, "layers_of_shape": full_layers, "hidden_size": H,
                    "num_attention_heads": Hq, "num_key_value_heads": Hkv, "head_dim": D, "intermediate_size": I,
                    "vocab_size": V, "kv_page_size": page, "prefill_tokens": T, "rope_theta": cfg.rope_theta,
-                   "rms_norm_eps": cfg.rms_norm_eps, "decode_graph": bool(not args.eager and hasattr(runner, "enable_decode_graphs")),
+                   "rms_norm_eps": cfg.rms_norm_eps, "decode_graph": not args.eager,
                    "decode_burst": 1 if args.eager else max(1, args.burst)},
         "prefill": {"value": round(T / pre_s, 1), "tokens": T, "ms": round(pre_s * 1e3, 3),
                     "frac": round(prefill_flops / pre_s / PEAK_FLOPS[args.dtype], 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4)},
-        "points": {f"decode_b{b}": round(results[b][0], 2) for b in points if b != args.batch},
+        "points": {**{f"decode_b{b}": round(results[b][0], 2) for b in points if b != args.batch}, **extra_points},
     }
+    if serve:
+        line[f"serve_{args.serve_seqs}"] = serve
     print(json.dumps(line), flush=True)
     return 0
 

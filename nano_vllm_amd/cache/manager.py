@@ -157,14 +157,20 @@ class CacheManager:
 
     def can_reserve_all(self, wanted: Sequence[Tuple[Hashable, int, Optional[int]]]) -> bool:
         """Whether reserve() would succeed for every (request, new_len, first_query) of `wanted`,
-        one after the other: all of them, or none, is what a caller needs who must not keep
-        pages for some requests when others find none."""
-        need = [0] * len(self.pools)
+        one after the other in the order given: all of them, or none, is what a caller needs who
+        must not keep pages for some requests when others find none.  The free pages are counted
+        along as the calls would leave them: a request is credited the pages its own window has
+        passed (reserve gives them back before it takes), never those of a request after it."""
+        free = [pool.num_free for pool in self.pools]
         for request, new_len, first_query in wanted:
-            for g, (n, give) in enumerate(zip(self.pages_needed(request, new_len, first_query),
-                                              self._passed_pages(request, first_query))):
-                need[g] += n - give
-        return all(pool.num_free >= n for pool, n in zip(self.pools, need))
+            need = self.pages_needed(request, new_len, first_query)
+            give = self._passed_pages(request, first_query)
+            for g in range(len(free)):
+                free[g] += give[g]
+                if free[g] < need[g]:
+                    return False
+                free[g] -= need[g]
+        return True
 
     def _passed_pages(self, request, first_query) -> List[int]:
         rc = self.requests[request]

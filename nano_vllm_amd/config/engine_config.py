@@ -21,7 +21,7 @@ class EngineConfig:
     enforce_eager: bool = False             # True: never replay a captured decode graph
     eos: int = -1                           # -1: taken from config.json / generation_config.json
     kvcache_block_size: int = 256           # any positive size (the reference demands % 256)
-    num_kvcache_blocks: int = -1            # -1: sized from free device memory
+    num_kvcache_blocks: int = -1            # -1: sized from free device memory; a list: one count per cache group
     # beyond the reference
     dtype: Optional[str] = None             # None: config.json's; "bfloat16" or "float32"
     seed: int = 0                           # sampling seed
@@ -30,6 +30,7 @@ class EngineConfig:
     device: str = "cuda:0"
     decode_burst: int = 8                   # decode steps in a row without the host, while no request waits (1: never)
     random_weights: Optional[int] = None    # a seed: the folder needs config.json only, weights are drawn on the device
+    measure_products: bool = True           # False: product kernels for 17-256 rows by rule and record only, nothing is timed at start-up
 
     def __post_init__(self):
         if not os.path.isdir(self.model):                          # config.py:21

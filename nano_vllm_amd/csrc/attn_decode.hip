@@ -71,8 +71,6 @@ __device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf1
     for (int dt = 0; dt < DT; ++dt) vf[dt] = *reinterpret_cast<const bf16x8*>(pv + (int64_t)dt * 16 * vt);
 }
 
-// waves a CU holds at once: the kernel's registers allow two per SIMD, eight per CU
-#define DEC_WAVES_PER_CU 8
 #define DEC_MAX_TOKENS 1024        // tokens of one launch: one wave plans them, 16 to a lane
 
 // The plan of a step's decode attention, made on the device from the tokens' positions by one small
@@ -499,33 +497,50 @@ attn_decode_merge_wave_kernel(const float* __restrict__ part_o, const float* __r
     }
 }
 
-// Waves the current GPU holds at once (asked of the device once), or 0 after leaving a message.
-static int decode_resident_waves() {
-    static int resident = 0;
-    if (!resident) {
-        int dev = 0, cus = 0;
+// Waves of the attention kernel for this head size that the current GPU holds at once: the CUs of
+// the device times the workgroups (of one wave) of that instance a CU takes, both asked of the
+// runtime once.  0 after leaving a message.
+static int decode_resident_waves(int head_dim) {
+    static int resident[9];                 // by head_dim / 32
+    if (head_dim % 32 || head_dim < 32 || head_dim > 256) {
+        nva_fail("attn_decode: head_dim %d has no instance", head_dim);
+        return 0;
+    }
+    int& r = resident[head_dim / 32];
+    if (!r) {
+        int dev = 0, cus = 0, per_cu = 0;
         if (hipGetDevice(&dev) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
             nva_fail("attn_decode: cannot read the number of CUs");
             return 0;
         }
-        resident = DEC_WAVES_PER_CU * cus;
+        hipError_t e = hipSuccess;
+        switch (head_dim) {
+#define OCC(DD) case DD: e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, attn_decode_kernel<DD>, NVA_WAVE, 0); break
+            OCC(32); OCC(64); OCC(96); OCC(128); OCC(160); OCC(192); OCC(224); OCC(256);
+#undef OCC
+        }
+        if (e != hipSuccess || per_cu <= 0) {
+            nva_fail("attn_decode: cannot read how many waves a CU holds (%s)", hipGetErrorString(e));
+            return 0;
+        }
+        r = per_cu * cus;
     }
-    return resident;
+    return r;
 }
 
 // What the decode attention of `tokens` single tokens needs when no request holds more than `longest`
 // keys: the bound of the segments of all tokens together, the number of persistent waves (a multiple
 // of the kv heads), and the size of the plan (int32).  Partial results: max_segments * num_q_heads *
 // (head_dim + 2) floats.
-NVA_EXPORT int nva_attn_decode_plan_size_bf16(int longest, int64_t tokens, int num_kv_heads, int page_size,
+NVA_EXPORT int nva_attn_decode_plan_size_bf16(int longest, int64_t tokens, int num_kv_heads, int head_dim, int page_size,
                                               int* max_segments, int* waves, int64_t* plan_ints) {
     if (longest <= 0 || tokens <= 0 || tokens > DEC_MAX_TOKENS || num_kv_heads <= 0 || page_size <= 0 ||
         !max_segments || !waves || !plan_ints)
         return nva_fail("attn_decode_plan_size: bad arguments (at most %d tokens a launch)", DEC_MAX_TOKENS);
     // a token sees at most longest / 32 + 2 chunks (a window may begin and end inside a chunk)
     const int64_t chunks = tokens * ((int64_t)longest / DEC_CHUNK + 2);
-    const int resident = decode_resident_waves();
+    const int resident = decode_resident_waves(head_dim);
     if (!resident) return -1;
     int64_t per_head = resident / num_kv_heads > 0 ? resident / num_kv_heads : 1;
     if (per_head > (chunks + 1) / 2) per_head = (chunks + 1) / 2;           // a quota has at least two chunks
@@ -565,6 +580,11 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_decode: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
     const int G = num_q_heads / num_kv_heads;
+    if (!(scale > 0.f) || !(scale <= 3.0e38f)) {
+        // the running maximum is taken of the raw scores and the scale folded into the exponent
+        nva_fail("attn_decode: needs a positive, finite scale (got %g)", (double)scale);
+        return 1;
+    }
     if (G > 16 || head_dim % 32 || head_dim < 32 || head_dim > 256 || page_size % 8 || page_size <= 0) {
         nva_fail("attn_decode: needs head_dim %% 32 == 0 in 32..256, at most 16 query heads per kv head and "
                  "page_size %% 8 == 0 (got head_dim %d, group %d, page %d)", head_dim, G, page_size);
@@ -599,7 +619,7 @@ NVA_EXPORT int nva_attn_decode_bf16(const void* q, int64_t q_stride, void* out, 
     int rc = nva_check_launch("attn_decode");
     if (rc) return rc;
     const int64_t pairs = tokens * num_q_heads;
-    const int resident = decode_resident_waves();
+    const int resident = decode_resident_waves(head_dim);
     if (!resident) return -1;
     if (pairs >= 2 * resident) {            // pairs enough for a wave each
         hipLaunchKernelGGL(attn_decode_merge_wave_kernel, dim3((unsigned)((pairs + MERGE_WAVES - 1) / MERGE_WAVES)),

@@ -120,7 +120,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, int64_t q_stride, __bf16* __re
     const int ny = num_kv_heads * ((num_q_heads / num_kv_heads + PF_WAVES - 1) / PF_WAVES);
     int rank = blockIdx.x;
     if (paired) {
-        const int heavy = 8 * ((paired + 15) / 16);
+        const int heavy = NVA_XCDS * ((paired + 2 * NVA_XCDS - 1) / (2 * NVA_XCDS));
         if (rank >= heavy) rank = paired - 1 - (rank - heavy);
     }
     const int by = rank % ny;
@@ -540,6 +540,11 @@ NVA_EXPORT int nva_attn_prefill_bf16(const void* q, int64_t q_stride, void* out,
     if (num_tiles == 0) return 0;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads)
         return nva_fail("attn_prefill: %d query heads do not divide into %d kv heads", num_q_heads, num_kv_heads);
+    if (!(scale > 0.f) || !(scale <= 3.0e38f)) {
+        // the running maximum is taken of the raw scores and the scale folded into the exponent
+        nva_fail("attn_prefill: needs a positive, finite scale (got %g)", (double)scale);
+        return 1;
+    }
     if (head_dim % 32 || head_dim < 32 || head_dim > 256 || page_size % 8 || page_size <= 0) {
         nva_fail("attn_prefill: needs head_dim %% 32 == 0 in 32..256 and page_size %% 8 == 0 (got %d, %d)", head_dim,
                  page_size);

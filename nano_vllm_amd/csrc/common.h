@@ -26,6 +26,9 @@ typedef float elem_t;
 #endif
 
 #define NVA_WAVE 64
+// gfx950: the compute units are spread over this many dies (XCDs), each with an L2 of its own;
+// workgroups are handed to the dies in turn, in the order of their index.
+#define NVA_XCDS 8
 
 // ---------------------------------------------------------------------------- errors
 static thread_local char nva_error_text[512];

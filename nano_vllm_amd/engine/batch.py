@@ -9,12 +9,10 @@ sees (tokens in the cache after this step) and its block table per cache group.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Hashable, List, Optional, Sequence
+from typing import Callable, Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
 import torch
-
-from ..kernels.ops import prefill_tile_order
 
 
 @dataclass
@@ -44,7 +42,6 @@ class StepBatch:
     seq_starts: torch.Tensor         # int32 [S] tokens each request had in the cache before
     state_slots: torch.Tensor        # int32 [S]
     logits_rows: Optional[torch.Tensor]   # int32 [R] flat token indices, in the caller's order
-    prefill_tiles: Optional[torch.Tensor]  # int32 [tiles, 2]: (request, 32-row tile) of the portions, most keys first
     groups: List[GroupBatch]
     max_q_len: int
     max_kv_len: int
@@ -53,11 +50,15 @@ class StepBatch:
     starts: List[int] = field(default_factory=list)
     requests: List[Hashable] = field(default_factory=list)
     step_cache: dict = field(default_factory=dict)   # emptied by the model at the start of every pass
+    # int32 lists that the kernels asked to have uploaded with the batch (name -> device tensor);
+    # the batch builder does not know what they mean
+    extras: Dict[str, torch.Tensor] = field(default_factory=dict)
 
 
 def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size: int, device,
                 table_width: Optional[int] = None, static: Optional[torch.Tensor] = None,
-                pad_to: Optional[int] = None, max_position: Optional[int] = None) -> StepBatch:
+                pad_to: Optional[int] = None, max_position: Optional[int] = None,
+                extras: Optional[Callable[[List[int], List[int], int], Dict[str, List[int]]]] = None) -> StepBatch:
     """Orders the entries (single tokens first), checks them against the cache manager's
     block tables and uploads everything in one copy.
 
@@ -69,7 +70,10 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
     first entry that write nothing into the cache (slot -1): they read what the first request
     reads, and their logits, which follow the real ones, are dropped by the caller.
     max_position: the positions the model knows (rows of its position tables); an entry that
-    reaches beyond is refused here, since the kernels read those tables unchecked."""
+    reaches beyond is refused here, since the kernels read those tables unchecked.
+    extras(q_lens, starts, num_decode) -> {name: [int, ...]}: lists that depend on the step's
+    shape only and that the kernels want on the device; they travel in the same copy and come
+    back as StepBatch.extras[name] (flat int32)."""
     if not entries:
         raise ValueError("a step needs at least one entry")
     order = sorted(range(len(entries)), key=lambda i: (len(entries[i].tokens) != 1, i))
@@ -166,8 +170,10 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
         if max(widths, default=1) > table_width:
             raise ValueError(f"a block table of {max(widths)} pages exceeds the fixed width {table_width}")
         widths = [table_width] * num_groups
-    tile_order = prefill_tile_order(q_lens, starts, num_decode)
-    scalars = cu + kv_lens + starts + state_slots + rows + tile_order
+    extra_lists = dict(extras(q_lens, starts, num_decode)) if extras is not None else {}
+    scalars = cu + kv_lens + starts + state_slots + rows
+    for values in extra_lists.values():
+        scalars = scalars + list(values)
     if num_decode == S:                              # decoded tokens only: one list, one conversion
         flat: List[int] = one_ids + one_pos + list(range(S)) + scalars
         for g in range(num_groups):
@@ -207,14 +213,14 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
     b_ids, b_pos, b_seq = take(T), take(T), take(T)
     b_cu, b_kv, b_starts, b_slots = take(S + 1), take(S), take(S), take(S)
     b_rows = take(len(rows)) if rows else None
-    b_tiles = take(len(tile_order)).view(-1, 2) if tile_order else None
+    b_extras = {name: take(len(values)) for name, values in extra_lists.items()}
     groups = []
     for g in range(num_groups):
         sm = take(T)
         bt = take(S * widths[g]).view(S, widths[g])
         groups.append(GroupBatch(bt, sm))
     return StepBatch(
-        num_tokens=T, num_seqs=S, num_decode=num_decode, prefill_tiles=b_tiles,
+        num_tokens=T, num_seqs=S, num_decode=num_decode, extras=b_extras,
         input_ids=b_ids, positions=b_pos, token_seq=b_seq, cu_seqlens_q=b_cu, kv_lens=b_kv,
         seq_starts=b_starts, state_slots=b_slots, logits_rows=b_rows, groups=groups,
         max_q_len=max(q_lens), max_kv_len=max(kv_lens), q_lens=q_lens, starts=starts,

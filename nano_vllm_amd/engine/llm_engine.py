@@ -34,14 +34,15 @@ class LLMEngine:
         self.model = load_model(cfg.model, cfg.dtype, cfg.device, kernels, random_weights=cfg.random_weights)
         spec = self.model.spec
         cfg.max_model_len = min(cfg.max_model_len, spec.max_position)           # config.py:25
-        num_pages = cfg.num_kvcache_blocks
-        if num_pages is None or num_pages <= 0:
+        num_pages = cfg.num_kvcache_blocks          # one count for every cache group, or a list with one per group
+        if num_pages is None or (not isinstance(num_pages, (list, tuple)) and num_pages <= 0):
             num_pages = self._pages_from_free_memory()
             cfg.num_kvcache_blocks = num_pages
         self.runner = ModelRunner(self.model, cfg.kvcache_block_size, num_pages, cfg.max_num_seqs,
                                   enable_prefix_caching=cfg.enable_prefix_caching)
         if not cfg.enforce_eager and self.model.device.type == "cuda":
-            self.runner.enable_decode_graphs(min(cfg.max_num_seqs, 512), cfg.max_model_len)
+            self.runner.enable_decode_graphs(min(cfg.max_num_seqs, 512), cfg.max_model_len,
+                                             measure_products=cfg.measure_products)
             self.runner.capture_decode_graphs()          # at start-up, as the reference does (model_runner.py:222)
         eos = [cfg.eos] if cfg.eos >= 0 else list(spec.eos_token_ids) or self._eos_from_generation_config()
         self.tokenizer = None
@@ -54,34 +55,70 @@ class LLMEngine:
 
     # ------------------------------------------------------------------ set-up helpers
     def _pages_from_free_memory(self) -> int:
-        """As nanovllm/engine/model_runner.py:103-114: what gpu_memory_utilization of the
-        device leaves after the weights and a step's activations, in pages of all layers."""
+        """As nanovllm/engine/model_runner.py:91-114: the largest step the options allow is run
+        once (max_num_batched_tokens prompt tokens in requests of up to max_model_len), on a
+        cache just large enough for it, and the most device memory it held beside weights and
+        cache is measured; the pages are what gpu_memory_utilization of the device leaves after
+        everything in use now, that peak, and what the captured decode steps keep."""
         from ..cache import storage
         from ..cache.manager import plan_groups
         cfg, model = self.config, self.model
-        needs = model.cache_needs()
-        groups, _ = plan_groups(needs)
-        itemsize = torch.empty((), dtype=model.dtype).element_size()
-        per_page = sum(storage.bytes_per_page(needs, groups, cfg.kvcache_block_size, itemsize))
         if model.device.type != "cuda":
             raise RuntimeError("num_kvcache_blocks must be given when the model is not on a GPU")
+        needs = model.cache_needs()
+        groups, state_runs = plan_groups(needs)
+        itemsize = torch.empty((), dtype=model.dtype).element_size()
+        per_page = sum(storage.bytes_per_page(needs, groups, cfg.kvcache_block_size, itemsize))
+        step_peak = self._largest_step_peak()
+        torch.cuda.empty_cache()
         free, total = torch.cuda.mem_get_info(model.device)
         used = total - free
-        # activations of the largest step: a few rows of the widest intermediate per token
-        widest = max([model.spec.hidden_size] + [d.shape[0] for _, _, d in model.param_table.values()
-                                                  if len(d.shape) == 2 and d.shape[0] < model.spec.vocab_size])
-        activations = cfg.max_num_batched_tokens * (4 * widest + 8 * model.spec.hidden_size) * itemsize
-        activations += cfg.max_num_seqs * model.spec.vocab_size * 4 * 2
+        kept = 0
         if not cfg.enforce_eager:
             # every captured decode step keeps its own logits: one row per request of its batch size
             top = min(cfg.max_num_seqs, 512)
             rows = sum({ModelRunner.graph_batch_size(n) for n in range(1, top + 1)})
-            activations += rows * model.spec.vocab_size * 4
-        budget = int(total * cfg.gpu_memory_utilization) - used - activations
+            kept = rows * model.spec.vocab_size * 4
+        kept += cfg.max_num_seqs * storage.state_bytes_per_slot(needs, state_runs)
+        budget = int(total * cfg.gpu_memory_utilization) - used - step_peak - kept
         pages = budget // max(per_page, 1)
         if pages <= 0:
             raise RuntimeError("no device memory is left for the cache (model_runner.py:114)")
+        self.warmup_peak_bytes = step_peak
         return int(pages)
+
+    def _largest_step_peak(self) -> int:
+        """Bytes the largest step holds at its peak beyond what was allocated before it (weights and
+        cache): the step is run on a runner of its own whose cache holds just its tokens
+        (model_runner.py:91-101 runs it before the cache exists)."""
+        cfg, model = self.config, self.model
+        per_request = max(1, min(cfg.max_model_len - 1, cfg.max_num_batched_tokens))
+        lengths = []
+        left = cfg.max_num_batched_tokens
+        while left > 0 and len(lengths) < cfg.max_num_seqs:
+            lengths.append(min(per_request, left))
+            left -= lengths[-1]
+        page = cfg.kvcache_block_size
+        pages = sum((n + page - 1) // page for n in lengths)
+        runner = ModelRunner(model, page, pages, len(lengths), enable_prefix_caching=False)
+        try:
+            entries = []
+            for i, n in enumerate(lengths):
+                name = ("warm-up", i)
+                runner.cache.admit(name)
+                runner.cache.reserve(name, n)
+                entries.append(StepEntry(name, [0] * n, 0, [n - 1]))
+            torch.cuda.synchronize(model.device)
+            torch.cuda.reset_peak_memory_stats(model.device)
+            before = torch.cuda.memory_allocated(model.device)
+            logits = runner.step(entries)
+            Sampler(model.kernels, model.device).sample(logits, [1.0] * len(lengths), [0] * len(lengths), list(range(len(lengths))), lengths)
+            torch.cuda.synchronize(model.device)
+            peak = torch.cuda.max_memory_allocated(model.device) - before
+            del logits
+        finally:
+            del runner
+        return max(int(peak), 0)
 
     def _eos_from_generation_config(self) -> List[int]:
         path = os.path.join(self.config.model, "generation_config.json")
@@ -120,7 +157,8 @@ class LLMEngine:
     def step(self) -> Tuple[List[Tuple[int, List[int]]], int]:
         """One scheduling decision and one model step.  Returns the requests finished in it
         as (id, completion token ids), and the token count of the step: positive for a step
-        of prompt tokens, minus the number of requests for a decode step (llm_engine.py:49-55)."""
+        of prompt tokens, minus the number of decoded tokens for a decode step (llm_engine.py:49-55:
+        one per request; here times the steps of a burst)."""
         t0 = perf_counter()
         seqs, is_prefill = self.scheduler.schedule()
         num_tokens = 0
@@ -134,6 +172,7 @@ class LLMEngine:
                 if last:
                     sampled.append(seq)
             burst = self._burst_steps(seqs, entries, is_prefill)
+            decoded = len(seqs)                  # tokens a decode step reports: one per request and step of a burst
             if burst > 1:
                 rows = self.runner.decode_burst(
                     entries, burst, self.sampler, [s.temperature for s in seqs],
@@ -144,6 +183,7 @@ class LLMEngine:
                         s.num_scheduled_tokens = 1
                     self.scheduler.postprocess([s for s, _ in live], [t for _, t in live])
                     self.stats["decode_tokens"] += len(live)
+                decoded = len(seqs) * burst
                 self.stats["decode_tokens"] -= len(seqs)            # the first row is counted below
             else:
                 logits = self.runner.step(entries)
@@ -157,7 +197,7 @@ class LLMEngine:
                 elif self.model.device.type == "cuda":
                     torch.cuda.synchronize(self.model.device)
                 self.scheduler.postprocess(seqs, [tokens.get(s.seq_id, -1) for s in seqs])
-            num_tokens = sum(len(e.tokens) for e in entries) if is_prefill else -len(seqs)
+            num_tokens = sum(len(e.tokens) for e in entries) if is_prefill else -decoded
             dt = perf_counter() - t0
             # tokens by what they are (a mixed step holds both kinds), time by the kind of the step
             self.stats["prefill_tokens"] += sum(len(e.tokens) for e, d in zip(entries, decoding) if not d)

@@ -64,14 +64,15 @@ class ModelRunner:
         if self._graph_max_batch and self._graph_takes(entries):
             return self._step_graph(entries)
         batch = build_batch(entries, self.cache, self.page_size, self.model.spec.vocab_size, self.device,
-                            max_position=self.model.spec.max_position)
+                            max_position=self.model.spec.max_position,
+                            extras=getattr(self.kernels, "batch_extras", None))
         hidden = self.model.forward(batch, self.layer_caches)
         if batch.logits_rows is None:
             return None
         return self.model.logits(hidden, batch.logits_rows)
 
     # ------------------------------------------------------------------ captured decode steps
-    def enable_decode_graphs(self, max_batch: int, max_len: int) -> None:
+    def enable_decode_graphs(self, max_batch: int, max_len: int, measure_products: bool = True) -> None:
         """Decode steps (one token per request, its logits wanted) of up to max_batch requests
         and max_len cached tokens are captured as HIP graphs, one per padded batch size, at
         their first occurrence, and replayed from then on.  Reference: capture_cudagraph and
@@ -81,8 +82,9 @@ class ModelRunner:
             return          # a mixer with host-side state handling cannot be replayed blindly
         if max_len > self.model.spec.max_position:
             raise ValueError(f"decode graphs for {max_len} tokens: the model knows {self.model.spec.max_position} positions")
-        # which product kernel serves which row count of these steps: measured on the model's own weights
-        if self.device.type == "cuda" and hasattr(self.kernels, "choose_products"):
+        # which product kernel serves which row count of these steps: measured on the model's own
+        # weights, unless a record of an earlier measurement exists (or the caller wants the rules alone)
+        if measure_products and self.device.type == "cuda" and hasattr(self.kernels, "choose_products"):
             self.kernels.choose_products(self.model.params.values(), max_batch)
         self._graph_max_batch = max_batch
         self._graph_max_len = max_len

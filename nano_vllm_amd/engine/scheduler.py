@@ -56,10 +56,17 @@ class Scheduler:
                              f"{self.max_model_len}")
         # the prompt and one more token, group by group: a window group never holds the whole prompt
         need = self.cache.peak_pages(seq.num_tokens + 1, self.max_num_batched_tokens)
+        # A window group's need is known to the end: while the request decodes it holds the pages of
+        # one window, wherever that lies, however short the prompt was.  (The all-keys group grows
+        # with every token; what happens when it runs out is the scheduler's business, see above.)
+        final = min(seq.num_tokens + seq.max_tokens, self.max_model_len)
+        for g, pages in enumerate(self.cache.peak_pages(final, 1)):
+            if self.cache.groups[g].window is not None:
+                need[g] = max(need[g], pages)
         for g, (pages, pool) in enumerate(zip(need, self.cache.pools)):
             if pages > pool.num_pages:
-                raise ValueError(f"a prompt of {seq.num_tokens} tokens needs {pages} pages of cache group {g}; "
-                                 f"it has {pool.num_pages}")
+                raise ValueError(f"a prompt of {seq.num_tokens} tokens with up to {seq.max_tokens} more needs {pages} "
+                                 f"pages of cache group {g}; it has {pool.num_pages}")
         self.waiting.append(seq)
 
     # ------------------------------------------------------------------ one step's decision

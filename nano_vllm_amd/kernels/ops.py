@@ -116,6 +116,63 @@ def prefill_tile_order(q_lens, starts, first_seq: int) -> list:
     return [v for u in units for v in (u[1], u[2])]
 
 
+# What choose_products measured, per device name: {(n, k, gated): {ceil(rows / 16): "library" | "medium"}}.
+# One table per process and device, shared by every HipKernels there, and kept in a file beside the
+# compiled libraries, so that engines on the same model dispatch alike from one process to the next
+# (the two kernels round their sums differently).
+_product_choices: dict = {}
+
+
+def _choice_file(write: bool = False) -> Optional[str]:
+    """The record of the measured choices: named after the build of the product kernels it was
+    measured with, in the first folder for compiled libraries that holds one (write: that can take one)."""
+    import os
+    from . import build
+    lib = build.find_library("gemm_skinny", "bf16")
+    tag = os.path.basename(lib).split(".")[1] if lib else "unbuilt"
+    name = f"product_choice.{tag}.json"
+    for d in build.build_dirs():
+        path = os.path.join(d, name)
+        if os.path.isfile(path) or (write and build._writable(d)):
+            return path
+    return None
+
+
+def recorded_product_choices(device_name: str) -> dict:
+    table = _product_choices.get(device_name)
+    if table is None:
+        import json
+        table = _product_choices[device_name] = {}
+        path = _choice_file()
+        if path:
+            try:
+                with open(path) as f:
+                    stored = json.load(f).get(device_name, {})
+                for key, rows in stored.items():
+                    n, k, gated = key.split(",")
+                    table[(int(n), int(k), gated == "1")] = {int(r): c for r, c in rows.items() if c in ("library", "medium")}
+            except (OSError, ValueError, AttributeError):
+                table.clear()                   # an unreadable record is measured again
+    return table
+
+
+def _write_product_choices() -> None:
+    import json
+    import os
+    path = _choice_file(write=True)
+    if not path:
+        return
+    stored = {dev: {f"{n},{k},{int(g)}": {str(r): c for r, c in sorted(rows.items())} for (n, k, g), rows in table.items()}
+              for dev, table in _product_choices.items()}
+    tmp = f"{path}.{os.getpid()}.tmp"
+    try:
+        with open(tmp, "w") as f:
+            json.dump(stored, f, indent=1, sort_keys=True)
+        os.replace(tmp, path)
+    except OSError:
+        pass                                    # the record is a convenience: without it the next process measures again
+
+
 class HipKernels:
     """Every device operation of the engine.  Needs a GPU and the compiled libraries."""
 
@@ -135,22 +192,31 @@ class HipKernels:
         # bit 2: the decode attention's plan outgrew its bound
         self.fault_flag = torch.zeros(1, dtype=torch.int32, device=self.device)
         # Rows up to which the bfloat16 product runs on the engine's own kernels.
+        props = torch.cuda.get_device_properties(self.device)
+        cus = props.multi_processor_count
         self.own_matmul_rows = 16           # bfloat16 products with more rows go to the library ...
         self.skinny_max_rows = 64           # ... unless the weight is small (see _own_rows); the kernel's limit
         self.small_weight_bytes = 64 << 20
         self.medium_max_rows = 224          # rows of x the kernel for medium row counts is used for (it takes 256)
-        self.medium_max_weight_rows = 8192  # and the widest weight it is used for
         self.medium_row_tiles = 2           # 1: one block of 16 weight rows per wave in the kernel for up to 256 rows (tests)
         self.medium_shape = None            # (waves, row tiles, ranges of k) forced on that kernel (tests)
-        self.medium_target_workgroups = torch.cuda.get_device_properties(self.device).multi_processor_count   # one workgroup per CU
+        self.medium_target_workgroups = cus  # one workgroup per CU
         self.team_max_rows = 16             # rows of x of the kernel whose waves split k inside a workgroup, for wide weights
-        self.team_min_weight_rows = 8192    # the narrowest weight it is used for (qkv of an 8B model; o and down stay split over workgroups)
-        self.teams = torch.cuda.get_device_properties(self.device).multi_processor_count   # one workgroup per CU
+        # A weight is wide when every CU's team gets two blocks of 16 rows at least: with one block a
+        # team loads its x for that block alone and keeps nothing, and a weight with fewer blocks than
+        # twice the CUs leaves CUs idle or unevenly loaded; such a weight is split over k instead.
+        self.team_min_weight_rows = 2 * 16 * cus
+        self.medium_max_weight_rows = self.team_min_weight_rows   # the widest weight the rule gives to the kernel for up to 256 rows
+        self.teams = cus                    # one workgroup per CU
         self.skinny_waves_per_tile = 0      # waves of a workgroup that share rows of the weight and split k; 0: by rows of x
-        self.skinny_target_waves = 4096     # the k range of a few-row product is split until this many waves run
-        # (n, k, gated) -> {ceil(rows / 16): "library" | "medium"}: what choose_products measured
-        # for the model's own weights; where it has no entry the rules of _own_kernel decide
-        self.product_choice = {}
+        # the k range of a few-row product is split until this many waves run: as many as the GPU
+        # holds at four per SIMD (many short waves stream faster than few long ones)
+        self.skinny_target_waves = 16 * cus
+        # (n, k, gated) -> {ceil(rows / 16): "library" | "medium"}: what choose_products measured on
+        # this kind of device, in this process or an earlier one; where it has no entry the rules of
+        # _own_kernel decide.  Every HipKernels of the process shares the table.
+        self.product_choice = recorded_product_choices(props.name)
+        self.choice_margin = 0.10           # the rule's kernel stays unless the other is faster by more than this
         self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
         self.mfma_attention = True
@@ -364,20 +430,30 @@ class HipKernels:
         if measured is not None and (m + 15) // 16 in measured:
             choice = measured[(m + 15) // 16]
             return None if choice == "library" else choice
+        return self._rule_kernel(m, n, k)
+
+    def _rule_kernel(self, m: int, n: int, k: int) -> Optional[str]:
+        """The unmeasured answer of _own_kernel beyond 16 rows."""
         if m <= self.medium_max_rows and n <= self.medium_max_weight_rows:
             return "medium"
         if m <= self.skinny_max_rows and 2 * n * k <= self.small_weight_bytes:
             return "skinny"
         return None
 
-    def choose_products(self, tensors, max_rows: int, min_elements: int = 1 << 22, reps: int = 3) -> dict:
+    def choose_products(self, tensors, max_rows: int, min_elements: int = 1 << 22, reps: int = 3,
+                        remeasure: bool = False, record: bool = True) -> dict:
         """Measures, for every shape of weight among `tensors` (2-D bfloat16 of at least min_elements
         elements and at most 65536 rows: the layers' projections) and every row count that a captured
         decode step of up to max_rows requests can have beyond 16 (multiples of 16, at most 256),
         the library product against the engine's kernel for up to 256 rows, plain (as a norm or the
-        q/k preparation consumes it) and with the SwiGLU gating, and keeps the fastest per shape and
-        row count in self.product_choice.  The weights of one shape (one per layer) are used in
-        turn, so that none is found in a cache.  Returns what it chose."""
+        q/k preparation consumes it) and with the SwiGLU gating, and keeps the faster per shape and
+        row count in self.product_choice; the kernel that the rules of _own_kernel name stays unless
+        the other is faster by more than choice_margin, so that two near-equal candidates do not
+        swap from one measurement to the next.  The weights of one shape (one per layer) are used in
+        turn, so that none is found in a cache.  What was measured before, in this process or in one
+        that left its record beside the compiled libraries, is not measured again (remeasure: is),
+        so engines on the same model dispatch alike; record=False leaves that file alone.  Returns
+        the table."""
         import torch.nn.functional as F
         by_shape = {}
         for t in tensors:
@@ -386,7 +462,7 @@ class HipKernels:
                 by_shape.setdefault(tuple(t.shape), []).append(t)
         rows = [m for m in range(32, min(max_rows, MEDIUM_KERNEL_ROWS) + 1, 16)]
         if not by_shape or not rows:
-            return {}
+            return self.product_choice
         start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
 
         def timed(fn, weights) -> float:
@@ -398,14 +474,17 @@ class HipKernels:
             stop.synchronize()
             return start.elapsed_time(stop)
 
+        measured = False
         for (n, k), weights in by_shape.items():
             if not self._skinny_takes(weights[0], k, weights[0], k, k):
                 continue
             for gated in (False, True):
                 if gated and n % 2:
                     continue
-                table = {}
+                table = {} if remeasure else dict(self.product_choice.get((n, k, gated), {}))
                 for m in rows:
+                    if m // 16 in table:
+                        continue
                     x = torch.randn((m, k), dtype=torch.bfloat16, device=weights[0].device)
                     out = torch.empty((m, n // 2 if gated else n), dtype=torch.bfloat16, device=x.device)
                     cands = {}
@@ -417,8 +496,13 @@ class HipKernels:
                         cands["medium"] = lambda w: self._linear_medium(x, k, w, k, None, None, 0, False, False, m, n, k, defer=True)
                     # the smaller of two measurements each: a start-up has other work going on
                     times = {name: min(timed(fn, weights), timed(fn, weights)) for name, fn in cands.items()}
-                    table[m // 16] = min(times, key=times.get)
+                    usual = "medium" if self._rule_kernel(m, n, k) == "medium" else "library"
+                    other = "library" if usual == "medium" else "medium"
+                    table[m // 16] = other if times[other] < (1.0 - self.choice_margin) * times[usual] else usual
+                    measured = True
                 self.product_choice[(n, k, gated)] = table
+        if measured and record:
+            _write_product_choices()
         return self.product_choice
 
     @staticmethod
@@ -656,12 +740,14 @@ class HipKernels:
         # tokens [0, num_decode) are single decoded tokens: the matrix-core decode kernel takes
         # them where its shape limits allow; everything else runs the general kernel
         start = 0
-        if q.dtype == torch.bfloat16 and batch.num_decode > 0 and self.mfma_attention and \
+        # (the matrix-core kernels fold the scale into the exponent, which needs it positive)
+        mfma = self.mfma_attention and q.dtype == torch.bfloat16 and 0.0 < scale < float("inf")
+        if batch.num_decode > 0 and mfma and \
                 self._decode_kernel_takes(num_heads // num_kv_heads, head_dim, page_size, q, qs, out, os_):
             start = batch.num_decode
             self._attention_decode(q, qs, out, os_, k_cache, v_cache, tables, batch, start, num_heads, num_kv_heads,
                                    head_dim, page_size, scale, window)
-        if start < tokens and q.dtype == torch.bfloat16 and self.mfma_attention and start == batch.num_decode and \
+        if start < tokens and mfma and start == batch.num_decode and \
                 self._prefill_kernel_takes(head_dim, page_size, tables.shape[1], q, qs, out, os_):
             # portions of prompts: the matrix-core prefill kernel, one workgroup per 32 query rows
             tiles = self._prefill_tiles(batch, q.device)
@@ -691,19 +777,32 @@ class HipKernels:
         return out
 
     @staticmethod
+    def batch_extras(q_lens, starts, num_decode) -> dict:
+        """What these kernels want uploaded with a step's batch, from the step's shape alone (lengths
+        and starts of the requests' portions, single tokens first): the order in which the prefill
+        attention takes its tiles of 32 query rows.  Returned as {name: list of int}."""
+        if num_decode == len(q_lens):
+            return {}
+        return {"prefill_tiles": prefill_tile_order(q_lens, starts, num_decode)}
+
+    @staticmethod
     def _prefill_tiles(batch, device) -> torch.Tensor:
         """int32 [tiles, 2] = (request, tile of 32 query rows) of the step's portions of prompts, from the
-        most keys to the fewest; a batch that was not built by the engine gets them here, once."""
-        tiles = getattr(batch, "prefill_tiles", None)
+        most keys to the fewest: uploaded with the batch where the batch's builder was given
+        batch_extras, else made here, once per batch."""
+        extras = getattr(batch, "extras", None)
+        if extras is None:
+            extras = batch.extras = {}
+        tiles = extras.get("prefill_tiles")
         if tiles is None:
             flat = prefill_tile_order(batch.q_lens, batch.starts if getattr(batch, "starts", None) else
                                       [int(kv) - n for kv, n in zip(batch.kv_lens.tolist(), batch.q_lens)],
                                       batch.num_decode)
-            tiles = torch.tensor(flat, dtype=torch.int32, device=device).view(-1, 2)
-            batch.prefill_tiles = tiles
-        if tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 2 or not tiles.is_contiguous():
+            tiles = torch.tensor(flat, dtype=torch.int32, device=device)
+            extras["prefill_tiles"] = tiles
+        if tiles.dtype != torch.int32 or tiles.numel() % 2 or not tiles.is_contiguous():
             raise KernelError("attention: prefill_tiles must be contiguous int32 [tiles, 2]")
-        return tiles
+        return tiles.view(-1, 2)
 
     @staticmethod
     def _decode_kernel_takes(group, head_dim, page_size, q, q_stride, out, out_stride) -> bool:
@@ -728,12 +827,12 @@ class HipKernels:
             plans = batch.step_cache = {}
         for t0 in range(0, n, 1024):
             t1 = min(n, t0 + 1024)
-            key = ("decode_plan", t0, num_kv_heads, page_size, window or 0)
+            key = ("decode_plan", t0, num_kv_heads, head_dim, page_size, window or 0)
             if key not in plans:
                 bound, waves, ints = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int64(0)
                 library.call("attn_decode", "bf16", "nva_attn_decode_plan_size", c_i32(batch.max_kv_len), c_i64(t1 - t0),
-                             c_i32(num_kv_heads), c_i32(page_size), ctypes.byref(bound), ctypes.byref(waves),
-                             ctypes.byref(ints))
+                             c_i32(num_kv_heads), c_i32(head_dim), c_i32(page_size), ctypes.byref(bound),
+                             ctypes.byref(waves), ctypes.byref(ints))
                 plan = torch.empty(ints.value, dtype=torch.int32, device=q.device)
                 library.call("attn_decode", "bf16", "nva_attn_decode_plan", _p(batch.positions[t0:t1]),
                              _p(batch.token_seq[t0:t1]), c_i64(t1 - t0),

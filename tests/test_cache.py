@@ -230,3 +230,26 @@ def test_reserving_for_several_requests_is_all_or_nothing():
     assert m.can_reserve("a", 12, 7) and m.can_reserve("b", 12, 7)
     assert m.pools[0].num_free == 1
     m.check()
+
+
+def test_reserving_for_several_requests_counts_pages_in_the_order_of_the_calls():
+    """A window group: b's window has passed two pages that reserve(b) would give back, but a comes
+    first and finds no page; the sums over both balance, the calls one after the other fail."""
+    m = CacheManager([CacheGroup(8, (0,))], 4, 6)
+    m.admit("a")
+    m.reserve("a", 8)                        # 2 pages
+    m.admit("b")
+    m.reserve("b", 16)                       # 4 pages; none is free now
+    assert m.pools[0].num_free == 0
+    # a query at position 16 with a window of 8 sees positions 9..16: b's pages 0 and 1 have been passed
+    wanted = [("a", 9, 8), ("b", 17, 16)]
+    assert m.pages_needed("a", 9, 8) == [1] and m._passed_pages("a", 8) == [0]
+    assert m.pages_needed("b", 17, 16) == [1] and m._passed_pages("b", 16) == [2]
+    assert not m.can_reserve_all(wanted)                 # a, first, would raise OutOfPages
+    with pytest.raises(OutOfPages):
+        m.reserve("a", 9, first_query=8)
+    assert m.can_reserve_all(wanted[::-1])               # b first gives two pages back and takes one, a the other
+    m.reserve("b", 17, first_query=16)
+    m.reserve("a", 9, first_query=8)
+    assert m.pools[0].num_free == 0
+    m.check()

@@ -74,3 +74,21 @@ def test_row_counts_choose_the_product_kernel():
     assert k._own_kernel(48, 5120, 25600) == "medium"            # no measurement for 48 rows: the rule
     assert k._own_kernel(64, 51200, 5120, gated=True) == "skinny" and k._own_kernel(64, 51200, 5120) is None
     assert k._own_kernel(8, 5120, 25600) == "skinny"             # up to 16 rows nothing is measured
+
+
+def test_the_record_of_measured_choices_survives_a_round_trip(tmp_path, monkeypatch):
+    from nano_vllm_amd.kernels import ops
+    record = tmp_path / "choices.json"
+    monkeypatch.setattr(ops, "_choice_file", lambda write=False: str(record) if write or record.exists() else None)
+    monkeypatch.setattr(ops, "_product_choices", {})
+    assert ops.recorded_product_choices("a GPU") == {}
+    ops.recorded_product_choices("a GPU")[(4096, 12288, False)] = {2: "medium", 14: "library"}
+    ops.recorded_product_choices("a GPU")[(24576, 4096, True)] = {4: "library"}
+    ops._write_product_choices()
+    monkeypatch.setattr(ops, "_product_choices", {})
+    assert ops.recorded_product_choices("a GPU") == {(4096, 12288, False): {2: "medium", 14: "library"},
+                                                     (24576, 4096, True): {4: "library"}}
+    assert ops.recorded_product_choices("another GPU") == {}
+    record.write_text("not json")
+    monkeypatch.setattr(ops, "_product_choices", {})
+    assert ops.recorded_product_choices("a GPU") == {}           # an unreadable record: measured again

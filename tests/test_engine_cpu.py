@@ -102,6 +102,35 @@ def test_a_padded_batch_of_decoded_tokens_reads_what_the_first_request_reads():
         build_batch([StepEntry("p", toks["p"][7:], 7, [])], r.cache, r.page_size, 256, "cpu", pad_to=2)
 
 
+def test_the_batch_builder_uploads_what_the_kernels_ask_for_and_knows_no_kernel():
+    """Lists that a kernel wants on the device for a step (the prefill attention's tile order is
+    one) are asked of the kernels object and travel in the batch's one copy; the builder itself
+    imports nothing of the kernels."""
+    import ast
+    import nano_vllm_amd.engine.batch as batch_module
+    from nano_vllm_amd.engine.batch import build_batch
+    tree = ast.parse(open(batch_module.__file__).read())
+    imported = [n.module or "" for n in ast.walk(tree) if isinstance(n, ast.ImportFrom)]
+    assert not any("kernels" in m for m in imported), imported
+    r = _runner("a", 16)
+    for rid, n in (("p", 9), ("q", 6)):
+        r.cache.admit(rid)
+        r.cache.reserve(rid, n)
+    asked = []
+
+    def extras(q_lens, starts, num_decode):
+        asked.append((list(q_lens), list(starts), num_decode))
+        return {"first": [7, 8, 9], "none": [], "second": [len(q_lens)]}
+
+    entries = [StepEntry("p", list(range(9)), 0, [8]), StepEntry("q", [3], 0, [0])]
+    b = build_batch(entries, r.cache, r.page_size, 256, "cpu", extras=extras)
+    assert asked == [([1, 9], [0, 0], 1)]                  # single tokens first
+    assert b.extras["first"].tolist() == [7, 8, 9] and b.extras["second"].tolist() == [2]
+    assert b.extras["none"].numel() == 0 and b.extras["first"].dtype == torch.int32
+    assert b.logits_rows.tolist() == [9, 0] and b.groups[0].slot_mapping.numel() == 10
+    assert build_batch(entries, r.cache, r.page_size, 256, "cpu").extras == {}
+
+
 def _llm(name, **kw):
     c = H.CONFIGS[name]
     opts = dict(kernels=TorchKernels(), device="cpu", dtype="float32", kvcache_block_size=c["page"],

@@ -116,6 +116,7 @@ def test_temperature_sampling_is_reproducible_and_independent_of_the_batch():
 def test_cache_sized_from_free_memory():
     llm = LLM(H.model_folder("d", "bfloat16"), gpu_memory_utilization=0.05, max_num_batched_tokens=64, max_num_seqs=4)
     assert llm.config.num_kvcache_blocks > 0 and llm.config.kvcache_block_size == 256
+    assert llm.warmup_peak_bytes > 0              # the largest step was run and measured
     out = llm.generate([[1, 2, 3]], SamplingParams(temperature=0.0, max_tokens=3), use_tqdm=False)
     assert len(out[0]["token_ids"]) == 3
 

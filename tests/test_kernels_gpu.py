@@ -242,7 +242,8 @@ def test_the_product_kernel_is_chosen_by_measurement_and_every_choice_is_right()
     n, k = 4096, 1024
     weights = [_rand((n, k), torch.bfloat16, 70 + i, 0.05) for i in range(3)]
     small = _rand((64, 64), torch.bfloat16, 75)                     # below min_elements: not measured
-    table = kern.choose_products(weights + [small, weights[0].float()], max_rows=80)
+    kern.product_choice = {}                                        # a table of its own, and no record of it
+    table = kern.choose_products(weights + [small, weights[0].float()], max_rows=80, record=False)
     assert set(table) == {(n, k, False), (n, k, True)}
     for gated in (False, True):
         assert set(table[(n, k, gated)]) == {2, 3, 4, 5} and set(table[(n, k, gated)].values()) <= {"library", "medium"}
@@ -259,6 +260,35 @@ def test_the_product_kernel_is_chosen_by_measurement_and_every_choice_is_right()
         got = kern.linear(x, weights[1], deferred=True)
         _close(got.tensor() if hasattr(got, "tensor") else got, want.float().to(torch.bfloat16), torch.bfloat16, str(forced))
     kern.check_faults()
+
+
+def test_the_measured_choice_is_kept_with_a_margin_and_recorded(tmp_path, monkeypatch):
+    """The rule's kernel stays unless the other one is faster by more than the margin; what was
+    chosen is written beside the compiled libraries and read by the next process (here: after the
+    process's table is emptied), which measures nothing again."""
+    import json
+    from nano_vllm_amd.kernels import HipKernels, ops
+    record = tmp_path / "product_choice.json"
+    monkeypatch.setattr(ops, "_choice_file", lambda write=False: str(record) if write or record.exists() else None)
+    monkeypatch.setattr(ops, "_product_choices", {})
+    kern = HipKernels(DEV, torch.bfloat16, quiet=True)
+    assert kern.product_choice == {}
+    n, k = 2048, 2048
+    weights = [_rand((n, k), torch.bfloat16, 80 + i, 0.05) for i in range(3)]
+    kern.choice_margin = 1.0                   # nothing is faster by 100 %: the rule's kernel (few weight rows: "medium") stays
+    table = kern.choose_products(weights, max_rows=48)
+    assert table[(n, k, False)] == {2: "medium", 3: "medium"} and table[(n, k, True)] == {2: "medium", 3: "medium"}
+    name = torch.cuda.get_device_properties(0).name
+    assert json.loads(record.read_text())[name][f"{n},{k},0"] == {"2": "medium", "3": "medium"}
+    # the next process: its table comes from the record, and rows it holds are not measured again
+    monkeypatch.setattr(ops, "_product_choices", {})
+    again = HipKernels(DEV, torch.bfloat16, quiet=True)
+    assert again.product_choice[(n, k, True)] == {2: "medium", 3: "medium"}
+    again.choice_margin = -1e9                 # a measurement now would flip every entry to the library
+    table = again.choose_products(weights, max_rows=64)
+    assert table[(n, k, False)][2] == "medium" and table[(n, k, False)][3] == "medium" and table[(n, k, False)][4] == "library"
+    assert json.loads(record.read_text())[name][f"{n},{k},0"]["4"] == "library"
+    assert HipKernels(DEV, torch.bfloat16, quiet=True).product_choice is again.product_choice     # one table per process
 
 
 def test_the_kernel_for_wide_weights_refuses_what_it_does_not_take():

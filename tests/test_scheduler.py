@@ -225,3 +225,24 @@ def test_admission_is_sized_group_by_group():
         small.add(_seq(40))
     with pytest.raises(ValueError, match="cache group 0"):
         Scheduler(CacheManager(groups, 4, [8, 4], enable_prefix_caching=False), 4, 8, 64, (), "prefill_first").add(_seq(40))
+
+
+def test_a_short_prompt_that_decodes_across_the_window_is_sized_for_the_window():
+    """The window group's need while decoding (a whole window, at any offset) is checked when the
+    request is added, not found out later as cache_full: a prompt of 3 tokens fits one page, but
+    its 30 decoded tokens need the pages of a window of 10."""
+    groups = [CacheGroup(None, (0,)), CacheGroup(10, (1,))]
+    # 10 positions at any offset touch 4 pages of 4 (the worst: a window that starts on a page's last slot)
+    assert CacheManager(groups, 4, [16, 4], enable_prefix_caching=False).peak_pages(33, 1) == [9, 4]
+    with pytest.raises(ValueError, match="cache group 1"):
+        Scheduler(CacheManager(groups, 4, [16, 3], enable_prefix_caching=False), 4, 8, 64, (), "prefill_first").add(
+            _seq(3, max_tokens=30))
+    s = Scheduler(CacheManager(groups, 4, [16, 4], enable_prefix_caching=False), 4, 8, 64, (), "prefill_first")
+    q = _seq(3, max_tokens=30)
+    s.add(q)
+    _run(s)
+    assert q.finish_reason == "max_tokens" and q.num_completion_tokens == 30
+    assert s.cache.pools[1].num_free == 4
+    # a short answer never reaches the window's width: the same pool of 3 pages takes it
+    Scheduler(CacheManager(groups, 4, [16, 3], enable_prefix_caching=False), 4, 8, 64, (), "prefill_first").add(
+        _seq(3, max_tokens=4))

@@ -84,36 +84,116 @@ def test_order_shared_cache_and_window_groups(variant_folder, dtype):
     r.kernels.check_faults()
 
 
+@pytest.fixture(scope="module")
+def real_size_folder(tmp_path_factory):
+    """name -> folder of two layers with the layer sizes of a named Qwen3 shape (a smaller vocabulary
+    keeps the plain implementation quick), weights stored in bfloat16: the float32 engine and the
+    plain implementation widen the same numbers, so one folder serves both element types."""
+    from nano_vllm_amd.models.shapes import shape
+    folders = {}
+
+    def get(name):
+        if name not in folders:
+            cj = shape(name)
+            cj.update(num_hidden_layers=2, vocab_size=2048, max_position_embeddings=4096)
+            folders[name] = write_random_model(str(tmp_path_factory.mktemp(name) / "m"), cj, seed=5, dtype="bfloat16")
+        return folders[name]
+    return get
+
+
+# 8B: 32 heads in groups of four; 14B: 40 heads in groups of five, widths of 5120 and 17408;
+# 32B: 64 heads in groups of eight, 25600 inner channels: other instances of the product and
+# attention kernels than the 8B sizes run
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_layer_sizes_of_the_8b_shape(tmp_path, dtype):
-    """Two layers with the Qwen3-8B layer sizes (a smaller vocabulary keeps the plain
-    implementation quick): float32 against the plain implementation, whole, decoded and in
-    portions; bfloat16 against the plain implementation with bfloat16 roundings."""
-    cfg = Qwen3Config(vocab_size=2048, hidden_size=4096, num_hidden_layers=2, num_attention_heads=32,
-                      num_key_value_heads=8, head_dim=128, intermediate_size=12288, rms_norm_eps=1e-6,
-                      rope_theta=1000000.0, max_position_embeddings=4096, tie_word_embeddings=False)
-    folder = write_random_model(str(tmp_path / "m"), cfg, seed=5, dtype=dtype)
+@pytest.mark.parametrize("name", ["qwen3-8b", "qwen3-14b", "qwen3-32b"])
+def test_layer_sizes_of_the_named_shapes(real_size_folder, name, dtype):
+    """Two layers with the layer sizes of the benchmarks' shapes: float32 against the plain
+    implementation, whole, decoded and in portions; bfloat16 against the plain implementation with
+    bfloat16 roundings; then several requests in one step on a short pool."""
+    folder = real_size_folder(name)
     r = ModelRunner.from_folder(folder, dtype=dtype, page_size=256, num_pages=4, max_requests=2, quiet=True,
                                 enable_prefix_caching=False)
+    if dtype == "bfloat16":
+        # what an engine does at start-up: the product kernels for 17 to 256 rows are the ones the
+        # model's own weights choose, and those are the ones compared below
+        r.kernels.choose_products(r.model.params.values(), 256)
     n = 300                                   # crosses a page of 256
     toks = H.random_tokens(2048, n, 7)
     pcfg, w = plain.read_folder(folder)
-    want = plain.logits(w, pcfg, toks, None if dtype == "float32" else "bfloat16")
+    rounding = None if dtype == "float32" else "bfloat16"
+    want = plain.logits(w, pcfg, toks, rounding)
     tol = 2e-5 if dtype == "float32" else 2e-2
-    for portions in ([n], [n - 32] + [1] * 32, [250, 2, 7, 41], [100, 200]):       # 41, 100, 200 rows: the kernel for medium row counts
+    # 41, 100, 200, 241 rows: the kernels for medium row counts
+    for portions in ([n], [n - 32] + [1] * 32, [250, 2, 7, 41], [100, 200], [59, 241]):
         got = H.run_portions(r, "x", toks, portions)
         assert H.rel_err(got, want) < tol, portions
     r.kernels.check_faults()
-    del r
     # several requests in one step at these sizes: single tokens of three beside a portion of a
     # fourth, pages of 256, on a pool that holds three of the five requests
     lens = [300, 270, 40, 290, 180]
     reqs = {f"r{i}": H.random_tokens(2048, m, 20 + i) for i, m in enumerate(lens)}
+    choice = dict(getattr(r.kernels, "product_choice", {}))
+    del r
     r = ModelRunner.from_folder(folder, dtype=dtype, page_size=256, num_pages=5, max_requests=4, quiet=True,
                                 enable_prefix_caching=False)
+    if dtype == "bfloat16":
+        r.kernels.product_choice = choice
     got = H.run_mixed(r, reqs, seed=9)
     for rid, t in reqs.items():
-        want = plain.logits(w, pcfg, t, None if dtype == "float32" else "bfloat16")
-        assert H.rel_err(got[rid], want) < tol, rid
+        assert H.rel_err(got[rid], plain.logits(w, pcfg, t, rounding)) < tol, rid
     assert r.cache.pools[0].num_free == 5
     r.kernels.check_faults()
+
+
+def test_two_engines_on_one_model_choose_the_same_product_kernels(real_size_folder, tmp_path, monkeypatch):
+    """The product kernels for 17 to 256 rows are measured once and recorded: a second engine, and
+    a second process (its table emptied here, so that it comes from the record), run the same
+    kernels and give the same bfloat16 logits bit for bit at 17, 64 and 240 rows."""
+    from nano_vllm_amd.kernels import ops
+    record = tmp_path / "product_choice.json"
+    monkeypatch.setattr(ops, "_choice_file", lambda write=False: str(record) if write or record.exists() else None)
+    monkeypatch.setattr(ops, "_product_choices", {})
+    folder = real_size_folder("qwen3-8b")
+    toks = H.random_tokens(2048, 17 + 64 + 240, 31)
+
+    def logits_of_an_engine():
+        r = ModelRunner.from_folder(folder, dtype="bfloat16", page_size=256, num_pages=4, max_requests=2, quiet=True,
+                                    enable_prefix_caching=False)
+        r.enable_decode_graphs(256, 2048)           # measures, or finds the record
+        table = {key: dict(rows) for key, rows in r.kernels.product_choice.items()}
+        return H.run_portions(r, "x", toks, [17, 64, 240]), table
+
+    first, table = logits_of_an_engine()
+    assert record.exists() and (4096, 12288, False) in table and (24576, 4096, True) in table
+    assert all(set(rows) == set(range(2, 17)) for rows in table.values())
+    second, table2 = logits_of_an_engine()
+    monkeypatch.setattr(ops, "_product_choices", {})      # as in a new process
+    third, table3 = logits_of_an_engine()
+    assert table2 == table and table3 == table
+    assert torch.equal(first, second) and torch.equal(first, third)
+
+
+def test_the_cache_is_sized_from_the_measured_peak_of_the_largest_step(real_size_folder):
+    """nanovllm/engine/model_runner.py:91-114: the largest step is run once before the cache is
+    sized.  With 12 GiB granted beyond what is in use, a step of 16384 prompt tokens through the
+    engine stays inside the grant, and the grant is used: pages, weights and the measured peak fill it."""
+    from nano_vllm_amd import LLM, SamplingParams
+    folder = real_size_folder("qwen3-8b")
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    free, total = torch.cuda.mem_get_info()
+    in_use = total - free                         # other processes, and what earlier tests still hold
+    held_here = torch.cuda.memory_allocated()
+    grant = 12 << 30
+    llm = LLM(folder, dtype="bfloat16", gpu_memory_utilization=(in_use + grant) / total, max_num_batched_tokens=16384,
+              max_model_len=4096, max_num_seqs=8, enable_prefix_caching=False)
+    per_page = 2 * 2 * 8 * 128 * 256 * 2          # K and V, two layers, 8 kv heads of 128, pages of 256, bfloat16
+    cache_bytes = llm.config.num_kvcache_blocks * per_page
+    weights = sum(t.numel() * t.element_size() for t in llm.model.params.values())
+    assert llm.warmup_peak_bytes > 16384 * 4096 * 2 * 4       # a few rows of the width per token at the least
+    assert grant - (256 << 20) <= cache_bytes + weights + llm.warmup_peak_bytes + 15 * 2048 * 4 <= grant
+    torch.cuda.reset_peak_memory_stats()
+    prompts = [H.random_tokens(2048, 4095, 50 + i) for i in range(4)] + [H.random_tokens(2048, 4, 60)]
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=2), use_tqdm=False)
+    assert [len(o["token_ids"]) for o in outs] == [2] * 5 and llm.stats["steps"] <= 4      # all prompts in one step
+    assert torch.cuda.max_memory_allocated() - held_here <= grant
