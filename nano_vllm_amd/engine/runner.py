@@ -90,6 +90,7 @@ class ModelRunner:
         self._graph_max_len = max_len
         self._graph_table_width = (max_len + self.page_size - 1) // self.page_size
 
+    @torch.inference_mode()          # as step(): every capture of a process happens in the same mode
     def capture_decode_graphs(self) -> int:
         """Captures every batch size now, the largest first (so that the smaller ones find their
         memory in the shared pool), with stand-in requests of one token each; what cannot be
