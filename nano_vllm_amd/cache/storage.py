@@ -1,6 +1,7 @@
 """Device tensors of the cache: for every run of the model's order that keeps keys and
 values, K [pages, kv_heads, page, head_dim] and V [pages, kv_heads, page / vt, head_dim, vt]
-of its group's page count; for every run with fixed state, its tensors [slots, ...].
+of its group's page count; for every run with fixed state, its tensors [slots + 1, ...] (the
+last row belongs to no request: rows that pad a captured batch read and write it).
 
 Reference: nanovllm/engine/model_runner.py:103-121 keeps one tensor [2, layers, pages,
 page, kv_heads, head_dim].  Here a (page, kv head) block is contiguous, and V is stored
@@ -50,6 +51,7 @@ def allocate(needs, groups, state_runs, num_pages: Sequence[int], page_size: int
             caches[r] = LayerCache(group=g, k=k, v=v)
     for r in state_runs:
         caches[r] = LayerCache(state={
-            name: torch.zeros((max(num_slots, 1),) + tuple(shape), dtype=_state_dtype(dt), device=device)
+            # one row more than requests can hold: the slot of the rows that pad a captured batch
+            name: torch.zeros((num_slots + 1,) + tuple(shape), dtype=_state_dtype(dt), device=device)
             for name, (shape, dt) in needs[r].tensors.items()})
     return caches

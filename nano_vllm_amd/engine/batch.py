@@ -68,7 +68,8 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
     width the layout is the same for every step, which is what a captured graph replays on.
     pad_to (decoded tokens only) fills the batch up to that many requests with copies of the
     first entry that write nothing into the cache (slot -1): they read what the first request
-    reads, and their logits, which follow the real ones, are dropped by the caller.
+    reads, and their logits, which follow the real ones, are dropped by the caller; where requests
+    hold state slots, theirs is the spare slot after the requests' own.
     max_position: the positions the model knows (rows of its position tables); an entry that
     reaches beyond is refused here, since the kernels read those tables unchecked.
     extras(q_lens, starts, num_decode) -> {name: [int, ...]}: lists that depend on the step's
@@ -150,8 +151,11 @@ def build_batch(entries: Sequence[StepEntry], cache, page_size: int, vocab_size:
         pad = pad_to - S
         one_ids += [one_ids[0]] * pad
         one_pos += [one_pos[0]] * pad
-        for values in (kv_lens, starts, q_lens, state_slots):
+        for values in (kv_lens, starts, q_lens):
             values += [values[0]] * pad
+        # state: the spare slot that no request holds (the state tensors' last row), so that a mixer
+        # may read and write the padding rows' state like any other
+        state_slots += [cache.slots.num_slots if cache.slots.num_slots else state_slots[0]] * pad
         cu += list(range(S + 1, S + pad + 1))
         for g in range(num_groups):
             one_slots[g] += [-1] * pad

@@ -78,8 +78,8 @@ class ModelRunner:
         their first occurrence, and replayed from then on.  Reference: capture_cudagraph and
         the replay branch of run_model (nanovllm/engine/model_runner.py:195-212,222-257),
         which captures every size at start-up."""
-        if self.state_runs:
-            return          # a mixer with host-side state handling cannot be replayed blindly
+        if any(not self.model.blocks[self.model.order[i].layer].replays_state_steps for i in self.state_runs):
+            return          # a mixer that handles its state on the host cannot be replayed blindly
         if max_len > self.model.spec.max_position:
             raise ValueError(f"decode graphs for {max_len} tokens: the model knows {self.model.spec.max_position} positions")
         # which product kernel serves which row count of these steps: measured on the model's own
@@ -152,6 +152,12 @@ class ModelRunner:
                                 table_width=self._graph_table_width, static=static, pad_to=size_b,
                                 max_position=self.model.spec.max_position)
             batch.max_kv_len = self._graph_max_len        # launch shapes must cover every later step
+            # The set-up runs below are real steps of these requests.  For keys and values that is
+            # harmless (the replay writes the same numbers to the same slots again); per-request
+            # state would be advanced three times, so the rows of this batch are put back afterwards.
+            rows = batch.state_slots.long() if self.state_runs else None
+            saved = [{name: t.index_select(0, rows) for name, t in self.layer_caches[i].state.items()}
+                     for i in self.state_runs]
             side = torch.cuda.Stream(self.device)
             side.wait_stream(torch.cuda.current_stream(self.device))
             with torch.cuda.stream(side):                 # what is set up lazily is set up outside the capture
@@ -159,6 +165,9 @@ class ModelRunner:
                     self.model.logits(self.model.forward(batch, self.layer_caches), batch.logits_rows)
             torch.cuda.current_stream(self.device).wait_stream(side)
             torch.cuda.synchronize(self.device)
+            for i, kept in zip(self.state_runs, saved):
+                for name, t in kept.items():
+                    self.layer_caches[i].state[name].index_copy_(0, rows, t)
             graph = torch.cuda.CUDAGraph()
             if self._graph_pool is None:                  # one memory pool for all sizes: they run one at a time
                 self._graph_pool = torch.cuda.graph_pool_handle()

@@ -43,6 +43,13 @@ class BuildContext:
 class Part:
     """Base of mixers, feed-forwards, norms, position encodings and blocks."""
 
+    # A mixer with per-request state says True when its forward, for a step of single tokens,
+    # reads the step's metadata on the device only (batch.state_slots, batch.seq_starts, ... as
+    # tensors; no .tolist() or .item(), nothing decided on the host from their values): such a step
+    # can be captured once and replayed for other requests.  Rows that pad a captured batch carry a
+    # state slot of their own that no request holds (the state tensors' last row).
+    replays_state_steps = False
+
     def __init__(self, params: Mapping, build: BuildContext):
         self.params = dict(params)
         self.kernels = build.kernels

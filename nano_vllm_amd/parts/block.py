@@ -39,6 +39,10 @@ class PreNormResidualBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need()
 
+    @property
+    def replays_state_steps(self):
+        return self.mixer.replays_state_steps
+
     def forward(self, h, residual, batch, cache):
         if residual is None:
             x, residual = self.mixer_norm.forward(h), h

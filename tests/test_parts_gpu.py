@@ -274,6 +274,102 @@ def test_a_toy_mixer_with_state_is_registered_built_and_stepped(tmp_path):
     assert H.rel_err(lost, whole["a"][10:]) > 1e-3
 
 
+class ToyDecayMixerOnDevice(ToyDecayMixer):
+    """The same mixer with its single-token steps written on the device only: the state rows are
+    gathered by batch.state_slots, reset where batch.seq_starts is 0, advanced and scattered back,
+    with no value of the batch read on the host.  Such a step can be captured and replayed."""
+    replays_state_steps = True
+
+    def forward(self, x, batch, cache):
+        if batch.num_decode != batch.num_seqs:
+            return super().forward(x, batch, cache)
+        state = cache.state["s"]
+        rows = batch.state_slots.long()
+        old = state.index_select(0, rows) * (batch.seq_starts != 0).float()[:, None]
+        new = self.decay * old + x.float()
+        state.index_copy_(0, rows, new)
+        return (new @ self.weights["mix.weight"].float().T).to(x.dtype)
+
+
+def test_single_token_steps_of_a_mixer_with_state_on_the_device_are_captured_and_replayed(tmp_path):
+    """A model with per-request state decodes through captured steps when its mixer says that it
+    handles the state on the device: every replay equals the eager step, with a batch size that is
+    captured at its first occurrence (whose set-up runs must not advance the state), rows of
+    padding, eager portions of another request between the replays, and bursts on the device."""
+    from nano_vllm_amd.sampling.sampler import Sampler
+    register_part("mixer", "toy_decay", ToyDecayMixerOnDevice, replace=True)
+    register_architecture("ToyStateLM", lambda d: d, _toy_spec, replace=True)
+    cfg = {"architectures": ["ToyStateLM"], "hidden_size": 64, "vocab_size": 99, "inner": 72, "eps": 1e-5, "decay": 0.5,
+           "torch_dtype": "float32"}
+    folder = write_random_model(str(tmp_path / "toy"), cfg, seed=5, std=0.1)
+    eager = ModelRunner.from_folder(folder, dtype="float32", page_size=8, num_pages=32, max_requests=5, quiet=True)
+    graphed = ModelRunner.from_folder(folder, dtype="float32", page_size=8, num_pages=32, max_requests=5, quiet=True)
+    graphed.enable_decode_graphs(max_batch=4, max_len=128)
+    assert graphed._graph_max_batch == 4 and graphed.state_runs == [0, 2]
+    assert graphed.layer_caches[0].state["s"].shape[0] == 5 + 1           # the last row: the padding rows' slot
+    reqs = {f"r{i}": H.random_tokens(99, n, 40 + i) for i, n in enumerate((60, 50, 45))}
+    extra = H.random_tokens(99, 23, 77)
+    for r in (eager, graphed):
+        for rid, toks in reqs.items():
+            r.cache.admit(rid)
+            r.cache.reserve(rid, 12)
+            r.step([StepEntry(rid, toks[:12], 0, [])])
+    pos = {rid: 12 for rid in reqs}
+    live = list(reqs)
+    for step in range(16):
+        if step == 6:
+            live = live[:2]
+        if step == 11:
+            live = list(reqs)
+        outs = []
+        for r in (eager, graphed):
+            entries = []
+            for rid in live:
+                r.cache.reserve(rid, pos[rid] + 1)
+                entries.append(StepEntry(rid, [reqs[rid][pos[rid]]], pos[rid], [0]))
+            outs.append(r.step(entries).clone())
+            if step % 3 == 1:
+                r.cache.admit("x")
+                r.cache.reserve("x", len(extra))
+                r.step([StepEntry("x", extra, 0, [len(extra) - 1])])
+                r.cache.release("x")
+            torch.cuda.synchronize()
+        for rid in live:
+            pos[rid] += 1
+        assert torch.equal(outs[0], outs[1]), f"replay {step} differs from the eager step"
+    assert sorted(graphed._graphs) == [2, 4]
+    # bursts: sampled tokens fed back on the device, the state advanced by the replays
+    sampler_e, sampler_g = Sampler(eager.kernels, eager.device), Sampler(graphed.kernels, graphed.device)
+    temps, seeds, ids = [0.0, 0.9, 0.0], [3, 3, 3], [0, 1, 2]
+    last = {rid: reqs[rid][pos[rid]] for rid in reqs}
+    toks_e = {rid: [last[rid]] for rid in reqs}
+    for _ in range(9):
+        entries = []
+        for rid in reqs:
+            n = pos[rid] + len(toks_e[rid])
+            eager.cache.reserve(rid, n)
+            entries.append(StepEntry(rid, [toks_e[rid][-1]], n - 1, [0]))
+        out = sampler_e.sample(eager.step(entries), temps, seeds, ids, [pos[rid] + len(toks_e[rid]) for rid in reqs])
+        for rid, tok in zip(reqs, out):
+            toks_e[rid].append(tok)
+    toks_g = {rid: [last[rid]] for rid in reqs}
+    for n in (4, 5):
+        entries = []
+        for rid in reqs:
+            m = pos[rid] + len(toks_g[rid])
+            graphed.cache.reserve(rid, m + n - 1)
+            entries.append(StepEntry(rid, [toks_g[rid][-1]], m - 1, [0]))
+        for row in graphed.decode_burst(entries, n, sampler_g, temps, seeds, ids):
+            for rid, tok in zip(reqs, row):
+                toks_g[rid].append(tok)
+    assert toks_e == toks_g
+    # a mixer that handles its state on the host keeps the runner eager
+    register_part("mixer", "toy_decay", ToyDecayMixer, replace=True)
+    host = ModelRunner.from_folder(folder, dtype="float32", page_size=8, num_pages=16, max_requests=3, quiet=True)
+    host.enable_decode_graphs(max_batch=4, max_len=128)
+    assert host._graph_max_batch == 0
+
+
 # ------------------------------------------------------------------------------ toy feed-forward with routing,
 # ------------------------------------------------------------------------------ toy position encoding
 class ToyRoutedFeedForward(Part):
