@@ -32,6 +32,7 @@ MODULES: Dict[str, Tuple[str, Tuple[Optional[str], ...]]] = {
     "gemm": ("gemm.hip", ("bf16", "f32")),
     "gemm_skinny": ("gemm_skinny.hip", ("bf16",)),
     "gemm_team": ("gemm_team.hip", ("bf16",)),
+    "gemm_tile": ("gemm_tile.hip", ("bf16",)),
     "attn_decode": ("attn_decode.hip", ("bf16",)),
     "attn_prefill": ("attn_prefill.hip", ("bf16",)),
     "sample": ("sample.hip", (None,)),

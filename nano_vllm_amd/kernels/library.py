@@ -22,7 +22,7 @@ _LAST_ERROR_SYMBOL = {
     "attn_generic": "nva_attn_generic_last_error", "gemm": "nva_gemm_last_error",
     "sample": "nva_sample_last_error", "attn_decode": "nva_attn_decode_last_error",
     "gemm_skinny": "nva_gemm_skinny_last_error", "gemm_team": "nva_gemm_team_last_error",
-    "attn_prefill": "nva_attn_prefill_last_error",
+    "attn_prefill": "nva_attn_prefill_last_error", "gemm_tile": "nva_gemm_tile_last_error",
 }
 
 _loaded: Dict[Tuple[str, Optional[str]], ctypes.CDLL] = {}

@@ -98,6 +98,7 @@ def check_positions_fit(table: torch.Tensor, head_dim: int, max_position: Option
 
 
 MEDIUM_KERNEL_ROWS = 256    # rows of x that nva_linear_medium takes
+TILE_KERNEL_ROWS = 256      # rows of x up to which the LDS-tiled product streams a weight (one tile of rows)
 PREFILL_ROWS = 32       # query rows of one workgroup of the prefill attention kernel
 PREFILL_MAX_TABLE = 4096    # pages of a block-table row the prefill attention kernel stages in LDS
 GENERAL_TILED_MAX_HEAD_DIM = 128    # head sizes of nva_paged_attention_tiled
@@ -116,7 +117,7 @@ def prefill_tile_order(q_lens, starts, first_seq: int) -> list:
     return [v for u in units for v in (u[1], u[2])]
 
 
-# What choose_products measured, per device name: {(n, k, gated): {ceil(rows / 16): "library" | "medium"}}.
+# What choose_products measured, per device name: {(n, k, gated): {ceil(rows / 16): "library" | "medium" | "tile"}}.
 # One table per process and device, shared by every HipKernels there, and kept in a file beside the
 # compiled libraries, so that engines on the same model dispatch alike from one process to the next
 # (the two kernels round their sums differently).
@@ -150,7 +151,8 @@ def recorded_product_choices(device_name: str) -> dict:
                     stored = json.load(f).get(device_name, {})
                 for key, rows in stored.items():
                     n, k, gated = key.split(",")
-                    table[(int(n), int(k), gated == "1")] = {int(r): c for r, c in rows.items() if c in ("library", "medium")}
+                    table[(int(n), int(k), gated == "1")] = {int(r): c for r, c in rows.items()
+                                                            if c in ("library", "medium", "tile")}
             except (OSError, ValueError, AttributeError):
                 table.clear()                   # an unreadable record is measured again
     return table
@@ -212,11 +214,13 @@ class HipKernels:
         # the k range of a few-row product is split until this many waves run: as many as the GPU
         # holds at four per SIMD (many short waves stream faster than few long ones)
         self.skinny_target_waves = 16 * cus
-        # (n, k, gated) -> {ceil(rows / 16): "library" | "medium"}: what choose_products measured on
+        # (n, k, gated) -> {ceil(rows / 16): "library" | "medium" | "tile"}: what choose_products measured on
         # this kind of device, in this process or an earlier one; where it has no entry the rules of
         # _own_kernel decide.  Every HipKernels of the process shares the table.
         self.product_choice = recorded_product_choices(props.name)
         self.choice_margin = 0.10           # the rule's kernel stays unless the other is faster by more than this
+        self.tile_for_wide_weights = True   # False: the rule never names the LDS-tiled kernel (tests)
+        self.tile_shape = None              # (shape, stages, ranges) forced on the LDS-tiled kernel (tests)
         self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
         self.mfma_attention = True
@@ -363,7 +367,7 @@ class HipKernels:
                     raise KernelError("linear: output does not match")
                 self._linear_team(x, xs, weight, ws, bias, out, os_, 1 if out_float32 else 0, m, n, k)
                 return out
-            if out_float32 and m > self.own_matmul_rows:
+            if out_float32 and m > self.own_matmul_rows and own != "tile":
                 # logits of many places: the library product with a float result reads the weight
                 # once, where the streaming kernel would read it once per 64 rows
                 y = torch.mm(x, weight.t(), out_dtype=torch.float32)
@@ -376,7 +380,9 @@ class HipKernels:
                     out.copy_(y)
                     return out
                 return y
-            run = self._linear_medium if own == "medium" else self._linear_skinny
+            if own == "tile" and not self._tile_takes(x, xs, weight, ws, m, n, k):
+                own = None
+            run = self._linear_medium if own == "medium" else self._linear_tile if own == "tile" else self._linear_skinny
             if deferred and own and not out_float32 and out is None and self.fuse_split_sums:
                 return run(x, xs, weight, ws, bias, None, 0, False, False, m, n, k, defer=True)
             if own or out_float32:
@@ -385,8 +391,8 @@ class HipKernels:
                 om, on, os_ = _rows2d(out, "linear output")
                 if (om, on) != (m, n) or out.dtype != out_dtype:
                     raise KernelError("linear: output does not match")
-                if own == "medium":
-                    self._linear_medium(x, xs, weight, ws, bias, out, os_, out_float32, False, m, n, k)
+                if own in ("medium", "tile"):
+                    run(x, xs, weight, ws, bias, out, os_, out_float32, False, m, n, k)
                     return out
                 rows = self.skinny_max_rows      # more rows (logits of many places): that many at a time
                 for r0 in range(0, m, rows):
@@ -411,15 +417,16 @@ class HipKernels:
 
     def _own_kernel(self, m: int, n: int, k: int, gated: bool = False) -> Optional[str]:
         """Which of the engine's weight-streaming kernels takes a bfloat16 product of m rows with a
-        weight [n, k]: "team", "skinny", "medium", or None for the library product.  Up to 16 rows
-        the engine's own kernels are as fast or faster for every weight ("team" for wide weights,
+        weight [n, k]: "team", "skinny", "medium", "tile", or None for the library product.  Up to 16
+        rows the engine's own kernels are as fast or faster for every weight ("team" for wide weights,
         whose waves split k inside a workgroup; "skinny" otherwise).  Beyond that the answer
         depends on the weight's shape and on what the library's heuristics pick for it, so it is
         measured once for the model's own weights (choose_products); without a measurement the
-        rules below stand, which were measured on the layer shapes of an 8B model: up to 224 rows
-        the medium kernel wins for weights of few rows (the library has no split of k and leaves
-        most of the GPU idle there), and loses for wide ones (gate/up); small wide weights stay
-        with the skinny kernel up to 64 rows."""
+        rules of _rule_kernel stand: up to 224 rows the medium kernel for weights of few rows (the
+        library has no split of k and leaves most of the GPU idle there), up to 256 rows the
+        LDS-tiled kernel for wide ones (gate/up, the head), whose every workgroup takes all of k
+        and does the gating itself; small wide weights whose k is no multiple of 64 stay with the
+        skinny kernel up to 64 rows."""
         if m <= 0:
             return None
         if m <= self.team_max_rows and n >= self.team_min_weight_rows and k % 32 == 0:
@@ -436,6 +443,8 @@ class HipKernels:
         """The unmeasured answer of _own_kernel beyond 16 rows."""
         if m <= self.medium_max_rows and n <= self.medium_max_weight_rows:
             return "medium"
+        if m <= TILE_KERNEL_ROWS and k % 64 == 0 and n > self.medium_max_weight_rows and self.tile_for_wide_weights:
+            return "tile"           # a wide weight (gate/up, the head): every workgroup takes all of k
         if m <= self.skinny_max_rows and 2 * n * k <= self.small_weight_bytes:
             return "skinny"
         return None
@@ -491,14 +500,19 @@ class HipKernels:
                     if gated:
                         cands["library"] = lambda w: self.silu_mul(F.linear(x, w), out=out)
                         cands["medium"] = lambda w: self._linear_medium(x, k, w, k, None, out, n // 2, False, True, m, n, k)
+                        if self._tile_takes(x, k, weights[0], k, m, n, k):
+                            cands["tile"] = lambda w: self._linear_tile(x, k, w, k, None, out, n // 2, False, True, m, n, k)
                     else:
                         cands["library"] = lambda w: F.linear(x, w)
                         cands["medium"] = lambda w: self._linear_medium(x, k, w, k, None, None, 0, False, False, m, n, k, defer=True)
+                        if self._tile_takes(x, k, weights[0], k, m, n, k):
+                            cands["tile"] = lambda w: self._linear_tile(x, k, w, k, None, None, 0, False, False, m, n, k, defer=True)
                     # the smaller of two measurements each: a start-up has other work going on
                     times = {name: min(timed(fn, weights), timed(fn, weights)) for name, fn in cands.items()}
-                    usual = "medium" if self._rule_kernel(m, n, k) == "medium" else "library"
-                    other = "library" if usual == "medium" else "medium"
-                    table[m // 16] = other if times[other] < (1.0 - self.choice_margin) * times[usual] else usual
+                    usual = self._rule_kernel(m, n, k)
+                    usual = usual if usual in cands else "library"
+                    best = min(times, key=times.get)
+                    table[m // 16] = best if times[best] < (1.0 - self.choice_margin) * times[usual] else usual
                     measured = True
                 self.product_choice[(n, k, gated)] = table
         if measured and record:
@@ -593,6 +607,53 @@ class HipKernels:
             return SplitSum(self, scratch, used.value, m, n, bias)
         return out
 
+    @staticmethod
+    def _tile_takes(x, xs, weight, ws, m, n, k) -> bool:
+        """The limits of nva_linear_tile: k in chunks of 64, 32-bit offsets into both operands."""
+        return k % 64 == 0 and (m * xs + k) * 2 < 2 ** 32 and (n * ws + k) * 2 < 2 ** 32
+
+    def _tile_plan(self, m: int, n: int, k: int, gated: bool, may_split: bool):
+        """(shape, stages, ranges of k) of the LDS-tiled kernel: the tile of rows that holds all m (64,
+        128 or 256; beyond that 256 and a grid dimension), 128 rows of the weight, as many stages as
+        LDS holds, and, where the result may stay as partial sums, k cut into as many ranges as give
+        about one workgroup per CU."""
+        if self.tile_shape is not None:
+            return self.tile_shape
+        shape, stages = (1, 4) if m <= 64 else (2, 3) if m <= 128 else (3, 4)
+        tiles = ((n // 2 if gated else n) + (63 if gated else 127)) // (64 if gated else 128)
+        ranges = 1
+        if may_split and not gated:
+            ranges = max(1, min(self.teams // max(tiles, 1), k // 256))
+        return shape, stages, ranges
+
+    def _linear_tile(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k, defer=False):
+        """The LDS-tiled kernel for 17 rows and more (see _linear_skinny for the arguments)."""
+        gated = bool(swiglu and bias is None and not defer)
+        shape, stages, ranges = self._tile_plan(m, n, k, gated, may_split=not gated and not out_float32)
+        if swiglu and not gated:
+            raise KernelError("linear_tile: the gated form takes no bias and is never deferred")
+        if ranges == 1:
+            if defer:
+                defer = False
+                out = torch.empty((m, n), dtype=x.dtype, device=x.device)
+                os_ = n
+            mode = 2 if gated else 1 if out_float32 else 0
+            library.call("gemm_tile", "bf16", "nva_linear_tile", _p(x), c_i64(xs), _p(weight), c_i64(ws), _p(bias), _p(out),
+                         c_i64(os_), None, c_i32(mode), c_i64(m), c_i64(n), c_i64(k), c_i32(shape), c_i32(stages), c_i32(1),
+                         None, self._stream())
+            return out
+        scratch = torch.empty(ranges * m * n, dtype=torch.float32, device=x.device)
+        used = ctypes.c_int(0)
+        library.call("gemm_tile", "bf16", "nva_linear_tile", _p(x), c_i64(xs), _p(weight), c_i64(ws), None, None, c_i64(0),
+                     _p(scratch), c_i32(3), c_i64(m), c_i64(n), c_i64(k), c_i32(shape), c_i32(stages), c_i32(ranges),
+                     ctypes.byref(used), self._stream())
+        sums = SplitSum(self, scratch, used.value, m, n, bias)
+        if defer:
+            return sums
+        library.call("gemm_skinny", "bf16", "nva_linear_skinny_finish", _p(scratch), c_i32(used.value), _p(bias), _p(out),
+                     c_i64(os_), c_i32(1 if out_float32 else 0), c_i32(0), c_i64(m), c_i64(n), self._stream())
+        return out
+
     def _linear_team(self, x, xs, weight, ws, bias, out, os_, mode, m, n, k):
         """The kernel for wide weights and at most 16 rows.  mode: 0 elements, 1 float, 2 gated."""
         library.call("gemm_team", "bf16", "nva_linear_team", _p(x), c_i64(xs), _p(weight), c_i64(ws), _p(bias), _p(out),
@@ -611,9 +672,11 @@ class HipKernels:
         if x.dtype == torch.bfloat16 and weight.dtype == x.dtype and wk == k and n % 2 == 0 and \
                 self._skinny_takes(x, xs, weight, ws, k):
             own = self._own_kernel(m, n, k, gated=True)
-            if own in ("skinny", "medium"):
+            if own == "tile" and not self._tile_takes(x, xs, weight, ws, m, n, k):
+                own = None
+            if own in ("skinny", "medium", "tile"):
                 out = torch.empty((m, n // 2), dtype=x.dtype, device=x.device)
-                run = self._linear_skinny if own == "skinny" else self._linear_medium
+                run = self._linear_skinny if own == "skinny" else self._linear_medium if own == "medium" else self._linear_tile
                 run(x, xs, weight, ws, None, out, n // 2, False, True, m, n, k)
                 return out
             if m > self.own_matmul_rows and (n, k, True) in self.product_choice:

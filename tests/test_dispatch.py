@@ -61,18 +61,21 @@ def test_row_counts_choose_the_product_kernel():
     k.own_matmul_rows, k.skinny_max_rows, k.small_weight_bytes = 16, 64, 64 << 20
     k.medium_max_rows, k.medium_max_weight_rows = 224, 8192
     k.team_max_rows, k.team_min_weight_rows, k.product_choice = 16, 8192, {}
+    k.tile_for_wide_weights = True
     assert k._own_kernel(1, 4096, 4096) == "skinny" and k._own_kernel(16, 24576, 4096) == "team"
     assert k._own_kernel(16, 24576, 4104) == "skinny"            # k no multiple of 32
     assert k._own_kernel(17, 4096, 4096) == "medium" and k._own_kernel(224, 4096, 12288) == "medium"
     assert k._own_kernel(0, 4096, 4096) is None
-    assert k._own_kernel(240, 5120, 25600) is None and k._own_kernel(64, 51200, 5120) is None
+    assert k._own_kernel(240, 5120, 25600) is None and k._own_kernel(64, 51200, 5120) == "tile"
+    assert k._own_kernel(256, 24576, 4096) == "tile" and k._own_kernel(257, 24576, 4096) is None
+    assert k._own_kernel(64, 24576, 4104) is None                # k no multiple of 64
     # what was measured on the model's own weights goes before the rules, per 16 rows, plain and gated apart
     k.product_choice[(5120, 25600, False)] = {15: "medium", 16: "medium", 2: "library"}
     k.product_choice[(51200, 5120, True)] = {4: "skinny"}
     assert k._own_kernel(240, 5120, 25600) == "medium" and k._own_kernel(225, 5120, 25600) == "medium"
     assert k._own_kernel(32, 5120, 25600) is None and k._own_kernel(17, 5120, 25600) is None
     assert k._own_kernel(48, 5120, 25600) == "medium"            # no measurement for 48 rows: the rule
-    assert k._own_kernel(64, 51200, 5120, gated=True) == "skinny" and k._own_kernel(64, 51200, 5120) is None
+    assert k._own_kernel(64, 51200, 5120, gated=True) == "skinny" and k._own_kernel(64, 51200, 5120) == "tile"
     assert k._own_kernel(8, 5120, 25600) == "skinny"             # up to 16 rows nothing is measured
 
 

@@ -246,12 +246,12 @@ def test_the_product_kernel_is_chosen_by_measurement_and_every_choice_is_right()
     table = kern.choose_products(weights + [small, weights[0].float()], max_rows=80, record=False)
     assert set(table) == {(n, k, False), (n, k, True)}
     for gated in (False, True):
-        assert set(table[(n, k, gated)]) == {2, 3, 4, 5} and set(table[(n, k, gated)].values()) <= {"library", "medium"}
+        assert set(table[(n, k, gated)]) == {2, 3, 4, 5} and set(table[(n, k, gated)].values()) <= {"library", "medium", "tile"}
     x = _rand((40, k), torch.bfloat16, 76)
     want = x.double() @ weights[1].double().T
     gu = want.float().to(torch.bfloat16).float()
     gated_want = torch.nn.functional.silu(gu[:, :n // 2]) * gu[:, n // 2:]
-    for forced in (None, "library", "medium"):
+    for forced in (None, "library", "medium", "tile"):
         if forced:
             kern.product_choice = {(n, k, g): {b: forced for b in range(2, 6)} for g in (False, True)}
             assert kern._own_kernel(40, n, k) == (None if forced == "library" else forced)
@@ -284,10 +284,11 @@ def test_the_measured_choice_is_kept_with_a_margin_and_recorded(tmp_path, monkey
     monkeypatch.setattr(ops, "_product_choices", {})
     again = HipKernels(DEV, torch.bfloat16, quiet=True)
     assert again.product_choice[(n, k, True)] == {2: "medium", 3: "medium"}
-    again.choice_margin = -1e9                 # a measurement now would flip every entry to the library
+    again.choice_margin = -1e9                 # a measurement now keeps the fastest, whatever the rule says
     table = again.choose_products(weights, max_rows=64)
-    assert table[(n, k, False)][2] == "medium" and table[(n, k, False)][3] == "medium" and table[(n, k, False)][4] == "library"
-    assert json.loads(record.read_text())[name][f"{n},{k},0"]["4"] == "library"
+    assert table[(n, k, False)][2] == "medium" and table[(n, k, False)][3] == "medium"
+    assert table[(n, k, False)][4] in ("library", "medium", "tile")
+    assert json.loads(record.read_text())[name][f"{n},{k},0"]["4"] == table[(n, k, False)][4]
     assert HipKernels(DEV, torch.bfloat16, quiet=True).product_choice is again.product_choice     # one table per process
 
 
@@ -335,6 +336,76 @@ def test_the_kernel_for_medium_row_counts_in_every_form(hip, m, n, k, splits, wa
         _close(got.tensor() if hasattr(got, "tensor") else got, want.float().to(torch.bfloat16), torch.bfloat16)
     finally:
         kern.medium_shape = None
+    kern.check_faults()
+
+
+# tile shapes of nva_linear_tile: (rows of x, rows of W, fed by a fifth wave, places of its x ring)
+TILE_SHAPES = {0: (64, 128, True, 3), 1: (64, 128, True, 3), 2: (128, 128, True, 3), 3: (256, 128, True, 3),
+               4: (64, 256, True, 3), 5: (128, 128, False, 0), 6: (256, 128, False, 0), 7: (256, 256, False, 0)}
+
+
+@pytest.mark.parametrize("shape,stages", [(0, 2), (0, 8), (1, 4), (2, 3), (3, 4), (4, 3), (5, 3), (6, 2), (7, 2)])
+@pytest.mark.parametrize("m,n,k,ranges", [(64, 512, 1024, 1), (17, 200, 192, 2), (40, 4096, 4096, 8), (97, 72, 64, 1),
+                                          (256, 520, 1024, 3), (150, 200, 320, 1), (300, 136, 2048, 5), (700, 1000, 576, 1)])
+def test_the_lds_tiled_product_in_every_form(hip, m, n, k, ranges, shape, stages):
+    """Every tile shape of the LDS-tiled kernel (the four multiplying waves fed by a fifth, or
+    fetching for themselves), few and many stages, unsplit and split over k, plain (with a bias),
+    gated, as float and as partial sums; row and column counts that fill no tile, more rows than a
+    tile holds (the grid's third dimension), a k range shorter than the ring."""
+    from nano_vllm_amd.kernels import KernelError
+    kern = hip[torch.bfloat16]
+    x, w = _rand((m, k), torch.bfloat16, 43), _rand((n, k), torch.bfloat16, 44, 0.05)
+    b = _rand((n,), torch.bfloat16, 45)
+    want = x.double() @ w.double().T
+    kern.tile_shape = (shape, stages, ranges)
+    try:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+        kern._linear_tile(x, k, w, k, b, out, n, False, False, m, n, k)
+        _close(out, (want + b.double()).float().to(torch.bfloat16), torch.bfloat16)
+        out32 = torch.empty((m, n), dtype=torch.float32, device=DEV)
+        kern._linear_tile(x, k, w, k, None, out32, n, True, False, m, n, k)
+        _close(out32, want.float(), torch.float32)
+        got = kern._linear_tile(x, k, w, k, b, None, 0, False, False, m, n, k, defer=True)
+        assert (ranges > 1) == hasattr(got, "tensor")
+        _close(got.tensor() if hasattr(got, "tensor") else got, (want + b.double()).float().to(torch.bfloat16), torch.bfloat16)
+        if ranges == 1:
+            gated = torch.empty((m, n // 2), dtype=torch.bfloat16, device=DEV)
+            y = want.float().to(torch.bfloat16).float()
+            if shape == 0:                       # one column block per wave: no place for a gate and its up
+                with pytest.raises(KernelError, match="two column blocks"):
+                    kern._linear_tile(x, k, w, k, None, gated, n // 2, False, True, m, n, k)
+            else:
+                kern._linear_tile(x, k, w, k, None, gated, n // 2, False, True, m, n, k)
+                _close(gated, (torch.nn.functional.silu(y[:, :n // 2]) * y[:, n // 2:]).to(torch.bfloat16), torch.bfloat16)
+    finally:
+        kern.tile_shape = None
+    kern.check_faults()
+
+
+def test_the_lds_tiled_product_refuses_what_it_does_not_take(hip):
+    from nano_vllm_amd.kernels import KernelError
+    kern = hip[torch.bfloat16]
+    assert not kern._tile_takes(None, 4104, None, 4104, 32, 512, 4104)          # k no multiple of 64
+    assert not kern._tile_takes(None, 4096, None, 4096, 32, 600000, 4096)       # a weight beyond 32-bit offsets
+    x, w = _rand((32, 4104), torch.bfloat16, 46), _rand((9000, 4104), torch.bfloat16, 47, 0.05)
+    assert kern._own_kernel(32, 9000, 4104) is None
+    _close(kern.linear(x, w), (x.double() @ w.double().T).float().to(torch.bfloat16), torch.bfloat16)
+    kern.tile_shape = (3, 8, 1)                  # eight stages of the largest tile: more than LDS holds
+    try:
+        with pytest.raises(KernelError, match="do not fit LDS"):
+            kern._linear_tile(_rand((32, 128), torch.bfloat16, 48), 128, _rand((64, 128), torch.bfloat16, 49), 128, None,
+                              torch.empty((32, 64), dtype=torch.bfloat16, device=DEV), 64, False, False, 32, 64, 128)
+    finally:
+        kern.tile_shape = None
+    # the rule sends a wide weight's rows 17 to 256 to this kernel, plain, gated and as float logits
+    n, k = 9216, 512
+    assert n > kern.medium_max_weight_rows and kern._own_kernel(100, n, k) == "tile"
+    x, w = _rand((100, k), torch.bfloat16, 50), _rand((n, k), torch.bfloat16, 51, 0.05)
+    want = x.double() @ w.double().T
+    _close(kern.linear(x, w), want.float().to(torch.bfloat16), torch.bfloat16)
+    _close(kern.linear(x, w, out_float32=True), want.float(), torch.float32)
+    y = want.float().to(torch.bfloat16).float()
+    _close(kern.linear_silu_mul(x, w), (torch.nn.functional.silu(y[:, :n // 2]) * y[:, n // 2:]).to(torch.bfloat16), torch.bfloat16)
     kern.check_faults()
 
 
