@@ -619,7 +619,7 @@ class HipKernels:
         about one workgroup per CU."""
         if self.tile_shape is not None:
             return self.tile_shape
-        shape, stages = (1, 4) if m <= 64 else (2, 3) if m <= 128 else (3, 4)
+        shape, stages = (1, 3) if m <= 64 else (2, 3) if m <= 128 else (3, 4)     # (64 rows: two workgroups fit a CU)
         tiles = ((n // 2 if gated else n) + (63 if gated else 127)) // (64 if gated else 128)
         ranges = 1
         if may_split and not gated:

@@ -213,3 +213,32 @@ def test_trace_run_as_a_user_calls_it(tmp_path, dtype):
         got = torch.from_numpy(np.fromfile(out / f"{s}.f32", dtype="<f4").reshape(len(places), V))
         want = torch.stack([plain_logits[rid][p] for rid, p in places])
         assert H.rel_err(got, want) < TOL[dtype], (s, places)
+
+
+def test_a_bfloat16_model_with_norm_weights_stored_in_float32(tmp_path):
+    """A tensor stored in 32 bits stays so: norm weights that a checkpoint stores in float32 are
+    used unrounded by the bfloat16 kernels (block norms, final norm, per-head q/k norms), whole and
+    in portions with decoded tokens.  The weights are made so that rounding them would show: 1 + d
+    with |d| below half a bfloat16 step, which rounds to exactly 1."""
+    from safetensors.torch import load_file, save_file
+    from nano_vllm_amd.weights import write_random_model
+    c = H.CONFIGS["b"]
+    folder = write_random_model(str(tmp_path / "m"), c["cfg"], seed=31, norm_std=0.0, dtype="bfloat16")
+    file = os.path.join(folder, "model.safetensors")
+    tensors = load_file(file)
+    gen = torch.Generator().manual_seed(5)
+    norms = [k for k in tensors if "norm" in k]
+    assert len(norms) == 4 * 3 + 1
+    for k in norms:
+        d = (torch.rand(tensors[k].shape, generator=gen) - 0.5) * 2 ** -8        # |d| < 2^-9: rounds away in bfloat16
+        tensors[k] = (1.0 + d).float()
+        assert torch.equal(tensors[k].to(torch.bfloat16).float(), torch.ones_like(d))
+    save_file(tensors, file, metadata={"format": "pt"})
+    r = H.make_runner(folder, "bfloat16", c["page"], 64)
+    assert all(r.model.params[k].dtype == torch.float32 for k in norms)
+    assert r.model.params["model.layers.0.mlp.down_proj.weight"].dtype == torch.bfloat16
+    toks = H.random_tokens(c["cfg"].vocab_size, 120, 8)
+    want = H.plain_logits(folder, toks, "bfloat16")
+    for portions in (H.whole(120), H.last_one_by_one(120), H.changing_portions(120, 2)):
+        assert H.rel_err(H.run_portions(r, "x", toks, portions), want) < TOL["bfloat16"]
+    r.kernels.check_faults()
