@@ -379,11 +379,8 @@ NVA_EXPORT int nva_linear_tile_bf16(const void* x, int64_t x_stride, const void*
             case 2: LAUNCH_KERNEL((linear_tile_fed_kernel<BM, BN, WM, WN, SX, 2>), 320); break;                        \
             case 3: LAUNCH_KERNEL((linear_tile_fed_kernel<BM, BN, WM, WN, SX, 3>), 320); break;                        \
             case 4: LAUNCH_KERNEL((linear_tile_fed_kernel<BM, BN, WM, WN, SX, 4>), 320); break;                        \
-            case 5: LAUNCH_KERNEL((linear_tile_fed_kernel<BM, BN, WM, WN, SX, 5>), 320); break;                        \
-            case 6: LAUNCH_KERNEL((linear_tile_fed_kernel<BM, BN, WM, WN, SX, 6>), 320); break;                        \
-            case 7: LAUNCH_KERNEL((linear_tile_fed_kernel<BM, BN, WM, WN, SX, 7>), 320); break;                        \
             case 8: LAUNCH_KERNEL((linear_tile_fed_kernel<BM, BN, WM, WN, SX, 8>), 320); break;                        \
-            default: return nva_fail("linear_tile: 2 to 8 stages, not %d", stages);                                    \
+            default: return nva_fail("linear_tile: 2, 3, 4 or 8 stages are built for this tile, not %d", stages);                                    \
         }                                                                                                              \
     } while (0)
 #define SELF(BM, BN, WM, WN)                                                                                           \
@@ -391,8 +388,7 @@ NVA_EXPORT int nva_linear_tile_bf16(const void* x, int64_t x_stride, const void*
         switch (stages) {                                                                                              \
             case 2: LAUNCH_KERNEL((linear_tile_kernel<BM, BN, WM, WN, 2>), 256); break;                                \
             case 3: LAUNCH_KERNEL((linear_tile_kernel<BM, BN, WM, WN, 3>), 256); break;                                \
-            case 4: LAUNCH_KERNEL((linear_tile_kernel<BM, BN, WM, WN, 4>), 256); break;                                \
-            default: return nva_fail("linear_tile: 2 to 4 stages, not %d", stages);                                    \
+            default: return nva_fail("linear_tile: 2 or 3 stages are built for this tile, not %d", stages);                                    \
         }                                                                                                              \
     } while (0)
     switch (shape) {
