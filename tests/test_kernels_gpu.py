@@ -785,6 +785,49 @@ def test_products_of_drawn_shapes(hip, ref, seed):
     kern.check_faults()
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_the_lds_tiled_product_at_drawn_shapes(hip, seed):
+    """Rows, widths, depths (multiples of 64), tile shapes, stages and cuts of k drawn at random for
+    the LDS-tiled kernel: plain with a bias, float within the bound of its rounding, gated, and
+    the partial sums added up."""
+    rng = random.Random(5000 + seed)
+    shape = rng.randrange(8)
+    bm, bn, fed, sx = TILE_SHAPES[shape]
+    lds = lambda st: (sx * bm + st * bn) * 128 if fed else st * (bm + bn) * 128
+    stages = rng.choice([st for st in ((2, 3, 4, 8) if fed else (2, 3)) if lds(st) <= 160 * 1024])
+    m = rng.choice([rng.randint(17, 64), rng.randint(65, 256), rng.randint(257, 600)])
+    n = 2 * rng.choice([rng.randint(1, 150), rng.randint(500, 4500)])
+    k = 64 * rng.choice([rng.randint(1, 8), rng.randint(20, 90)])
+    ranges = rng.choice([1, 1, rng.randint(2, 9)])
+    kern = hip[torch.bfloat16]
+    x, w = _rand((m, k), torch.bfloat16, 5100 + seed), _rand((n, k), torch.bfloat16, 5200 + seed, 0.05)
+    b = _rand((n,), torch.bfloat16, 5300 + seed)
+    want = x.double() @ w.double().T
+    what = f"m {m} n {n} k {k} shape {shape} stages {stages} ranges {ranges}"
+    kern.tile_shape = (shape, stages, ranges)
+    try:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
+        kern._linear_tile(x, k, w, k, b, out, n, False, False, m, n, k)
+        _close(out, (want + b.double()).float().to(torch.bfloat16), torch.bfloat16, what)
+        out32 = torch.empty((m, n), dtype=torch.float32, device=DEV)
+        kern._linear_tile(x, k, w, k, None, out32, n, True, False, m, n, k)
+        bound = (x.double().abs() @ w.double().abs().T) * (math.sqrt(k) * 2.0 ** -23) + 1e-30
+        assert bool(((out32.double() - want).abs() <= bound).all()), what + " float result"
+        got = kern._linear_tile(x, k, w, k, None, None, 0, False, False, m, n, k, defer=True)
+        if hasattr(got, "tensor"):
+            sums = got.sums[:got.splits * m * n].view(got.splits, m, n).double().sum(0)
+            assert bool(((sums - want).abs() <= bound).all()), what + " partial sums"
+        if shape != 0:
+            kern.tile_shape = (shape, stages, 1)
+            gated = torch.empty((m, n // 2), dtype=torch.bfloat16, device=DEV)
+            kern._linear_tile(x, k, w, k, None, gated, n // 2, False, True, m, n, k)
+            y = want.float().to(torch.bfloat16).float()
+            _close(gated, (torch.nn.functional.silu(y[:, :n // 2]) * y[:, n // 2:]).to(torch.bfloat16), torch.bfloat16, what + " gated")
+    finally:
+        kern.tile_shape = None
+    kern.check_faults()
+
+
 @pytest.mark.parametrize("page,lens,q_lens,window", [
     (256, [40000, 12345, 257, 4096], [1, 1, 1, 1], None),           # long decoding: 157 pages in a table
     (16, [30000, 5000], [1, 1], None),                              # the same over small pages: splits capped by pages
