@@ -9,9 +9,11 @@ request is released and when a window has passed them, and are taken again from 
 the free list.
 
 Reference: nanovllm/engine/block_manager.py:26-120 (one group, all keys, prefix hashes).
-The prefix-hash reuse of the reference is kept for models whose only cache is one group of
-all keys; where a window or per-request state exists, a hashed page would not carry all a
-request needs, and hits are switched off.
+The prefix-hash reuse of the reference works over every group: a full page is registered under
+the chained hash of its tokens in each group's pool, and a new request leaves out as many leading
+pages as every group can still stand for (an all-keys group all of them, a window group those the
+first computed token looks at).  Where per-request state of fixed size exists, pages do not carry
+all a request needs, and hits are switched off.
 """
 from __future__ import annotations
 
@@ -35,7 +37,7 @@ class RequestCache:
     tables: List[List[int]]        # per group
     num_tokens: int = 0            # positions reserved so far
     state_slot: int = -1
-    # chain of prefix hashes of the full pages registered so far (group 0 only)
+    # chain of prefix hashes of the full pages registered so far (the same chain in every group)
     hashes: List[int] = field(default_factory=list)
 
 
@@ -79,8 +81,9 @@ class CacheManager:
         self.pools = [PagePool(n, page_size) for n in counts]
         self.slots = SlotPool(num_state_slots)
         self.has_state = has_state
-        self.prefix_caching = (enable_prefix_caching and not has_state and len(self.groups) == 1
-                               and self.groups[0].window is None)
+        # Keys of a prefix are the same whoever computed them; state of fixed size is not kept by
+        # prefix, so a model with such state computes every prompt whole.
+        self.prefix_caching = enable_prefix_caching and not has_state
         self.requests: Dict[Hashable, RequestCache] = {}
 
     # ------------------------------------------------------------------ requests
@@ -205,24 +208,37 @@ class CacheManager:
         rc.num_tokens = max(rc.num_tokens, new_len)
 
     # ------------------------------------------------------------------ prefix reuse
-    def match_prefix(self, tokens: Sequence[int]) -> Tuple[int, List[int]]:
-        """How many leading full pages of `tokens` are in the cache already, and which pages:
-        the chain of hashes is followed until the first miss.  The last page of a request is
-        never taken from the cache, so that at least one token is computed
+    def match_prefix(self, tokens: Sequence[int]) -> Tuple[int, List[List[int]]]:
+        """How many leading full pages of `tokens` need not be computed, and per group which
+        pages stand for them (-1 where a window group needs none).  The chain of hashes is followed
+        through every group's pool: n leading pages can be left out if every group that keeps all
+        keys still holds all n, and every window group those that the first computed token,
+        position n * page_size, still looks at; the largest such n is taken.  The last page of a
+        request is never taken from the cache, so that at least one token is computed
         (block_manager.py:62-68)."""
         if not self.prefix_caching:
-            return 0, []
-        pool, ps = self.pools[0], self.page_size
+            return 0, [[] for _ in self.groups]
+        ps = self.page_size
         num_pages = (len(tokens) + ps - 1) // ps
-        h, pages = -1, []
+        found: List[List[int]] = [[] for _ in self.groups]
+        h = -1
         for i in range(num_pages - 1):
             block = tokens[i * ps:(i + 1) * ps]
             h = chain_hash(block, h)
-            page = pool.lookup(h, block)
-            if page == -1:
+            pages = [pool.lookup(h, block) for pool in self.pools]
+            if any(p == -1 and group.window is None for p, group in zip(pages, self.groups)):
+                break                       # nothing beyond a page that an all-keys group has lost
+            if all(p == -1 for p in pages):
                 break
-            pages.append(page)
-        return len(pages), pages
+            for g, p in enumerate(pages):
+                found[g].append(p)
+        hits = 0
+        for n in range(len(found[0]), 0, -1):
+            if all(-1 not in found[g][self._first_needed_page(g, n * ps):n] for g in range(len(self.groups))):
+                hits = n
+                break
+        return hits, [[p if i >= self._first_needed_page(g, hits * ps) else -1 for i, p in enumerate(found[g][:hits])]
+                      for g in range(len(self.groups))]
 
     def can_admit(self, tokens: Sequence[int], first_step: Optional[int] = None) -> int:
         """-1 if the pages for all of `tokens` are not free, else the number of leading pages
@@ -232,9 +248,8 @@ class CacheManager:
         hits, pages = self.match_prefix(tokens)
         step_end = None if first_step is None else hits * self.page_size + first_step
         for g, pool in enumerate(self.pools):
-            need = self._wanted_pages(g, len(tokens), step_end)
-            if g == 0:
-                need -= sum(1 for p in pages if not pool.is_free(p))
+            need = self._wanted_pages(g, len(tokens), step_end) - hits
+            need += sum(1 for p in pages[g] if p >= 0 and pool.is_free(p))
             if pool.num_free < need:
                 return -1
         if self.slots.num_slots and not self.slots.num_free:
@@ -248,11 +263,13 @@ class CacheManager:
         hits, pages = self.match_prefix(tokens)
         rc = self.admit(request)
         try:
-            pool = self.pools[0]
+            for pool, table, shared in zip(self.pools, rc.tables, pages):
+                for page in shared:
+                    if page >= 0:
+                        pool.share(page)
+                    table.append(page)
             h = -1
-            for i, page in enumerate(pages):
-                pool.share(page)
-                rc.tables[0].append(page)
+            for i in range(hits):
                 h = chain_hash(tokens[i * self.page_size:(i + 1) * self.page_size], h)
                 rc.hashes.append(h)
             cached = hits * self.page_size
@@ -266,17 +283,20 @@ class CacheManager:
 
     def register_full_pages(self, request: Hashable, tokens: Sequence[int], computed: int) -> None:
         """After a step: pages of the request that are now wholly computed get their chained
-        hash, so that later requests find them (block_manager.py:110-120).  `computed` is the
-        number of the request's leading tokens whose keys are in the cache."""
+        hash in every group that still holds them, so that later requests find them
+        (block_manager.py:110-120).  `computed` is the number of the request's leading tokens
+        whose keys are in the cache."""
         if not self.prefix_caching:
             return
         rc = self.requests[request]
-        pool, ps = self.pools[0], self.page_size
+        ps = self.page_size
         for i in range(len(rc.hashes), computed // ps):
             block = tokens[i * ps:(i + 1) * ps]
             h = chain_hash(block, rc.hashes[-1] if rc.hashes else -1)
             rc.hashes.append(h)
-            pool.register(rc.tables[0][i], h, block)
+            for pool, table in zip(self.pools, rc.tables):
+                if i < len(table) and table[i] >= 0:
+                    pool.register(table[i], h, block)
 
     # ------------------------------------------------------------------ checks
     def check(self) -> None:

@@ -190,7 +190,7 @@ def run_mixed_with_prefix_reuse(runner: ModelRunner, requests: Dict[str, List[in
             toks = requests[rid]
             if cache.can_admit(toks) == -1:
                 break
-            _, pages = cache.match_prefix(toks)
+            pages = cache.match_prefix(toks)[1][0]
             for p in pages:
                 stats["hit_given_back" if cache.pools[0].is_free(p) else "hit_in_use"] += 1
             if not pages:

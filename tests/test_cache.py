@@ -194,11 +194,115 @@ def test_a_hit_on_a_free_page_still_takes_it():
     m.check()
 
 
-def test_prefix_caching_is_off_with_windows_or_state():
-    assert _manager(groups=(None, 8)).prefix_caching is False
+def test_prefix_caching_is_off_with_state_only():
+    assert _manager(groups=(None, 8)).prefix_caching is True
+    assert _manager(groups=(8,)).prefix_caching is True
     assert _manager(slots=2).prefix_caching is False
     assert _manager(prefix=False).prefix_caching is False
     assert _manager().prefix_caching is True
+
+
+def test_prefix_pages_of_a_window_group():
+    """An all-keys group beside a window of 6 keys, pages of 4: a request that starts at page n
+    looks back at positions 4n - 5 .. 4n - 1, so the window group has to stand for pages n - 2
+    and n - 1 only, and its earlier entries stay -1."""
+    m = _manager(pages=12, page=4, groups=(None, 6))
+    toks = list(range(100, 122))                        # 22 tokens: 5 full pages and two tokens
+    assert m.admit_with_prefix("a", toks) == 0
+    for done in (8, 16, 22):                            # in three steps, as portions of a prompt
+        m.reserve("a", 22, first_query=done - 8 if done < 22 else 16)
+        m.register_full_pages("a", toks, done)
+        m.check()
+    ta, wa = list(m.table("a", 0)), list(m.table("a", 1))
+    assert wa[:2] == [-1, -1] and all(p >= 0 for p in wa[2:])      # pages 0 and 1 were passed at position 16
+    # an equal prompt: five pages are left out; the window group shares pages 3 and 4
+    hits, pages = m.match_prefix(toks)
+    assert hits == 5 and pages[0] == ta[:5] and pages[1] == [-1, -1, -1, wa[3], wa[4]]
+    assert m.admit_with_prefix("b", toks) == 20
+    assert m.table("b", 0)[:5] == ta[:5] and m.table("b", 1)[:5] == [-1, -1, -1, wa[3], wa[4]]
+    assert m.pools[1].ref_count[wa[4]] == 2 and m.pools[1].ref_count[wa[2]] == 1
+    m.check()
+    m.release("a")
+    m.check()
+    assert m.pools[1].ref_count[wa[4]] == 1
+    m.release("b")
+    m.check()
+    assert all(pool.num_free == pool.num_pages for pool in m.pools)
+    # the pages that a's window had passed went back first and are findable still
+    # (nothing has taken them): a prompt cut after two pages finds both groups' pages 0 and 1
+    assert m.can_admit(toks[:9]) == 2
+
+
+def test_a_window_page_that_is_gone_shortens_the_hit():
+    m = _manager(pages=12, page=4, groups=(None, 6))
+    toks = list(range(100, 122))
+    m.admit_with_prefix("a", toks)
+    m.register_full_pages("a", toks, 22)
+    wa = list(m.table("a", 1))
+    m.release("a")
+    assert m.can_admit(toks) == 5
+    # window page 3 is taken again by another request: hits that need it (n = 4 and 5) are gone,
+    # n = 3 needs window pages 1 and 2 only
+    pool = m.pools[1]
+    while pool.hash_to_page.get(pool.hash_of[wa[3]]) == wa[3]:
+        pool.take()
+    hits, pages = m.match_prefix(toks)
+    taken = [p for p in range(pool.num_pages) if pool.ref_count[p]]
+    for p in taken:
+        pool.give_back(p)
+    assert hits == 3 and pages[1] == [-1, wa[1], wa[2]] and len(pages[0]) == 3
+    # an all-keys page that is gone ends the chain there
+    m2 = _manager(pages=12, page=4, groups=(None, 6))
+    m2.admit_with_prefix("a", toks)
+    m2.register_full_pages("a", toks, 22)
+    t2 = list(m2.table("a", 0))
+    m2.release("a")
+    m2.pools[0].tokens_of[t2[2]] = (0, 0, 0, 0)
+    assert m2.can_admit(toks) == 2
+
+
+def test_random_requests_with_shared_prefixes_over_two_groups():
+    """Requests drawn from a few common prefixes come and go in random order on small pools of
+    an all-keys and a window group: the books balance after every call, a hit never exceeds what
+    was registered, and at the end every page is free."""
+    rng = random.Random(5)
+    page, window = 4, 10
+    m = _manager(pages=40, page=page, groups=(None, window))
+    stems = [[rng.randrange(50) for _ in range(rng.randrange(8, 40))] for _ in range(3)]
+    live = {}
+    hits_seen = 0
+    for i in range(400):
+        if live and (len(live) >= 4 or rng.random() < 0.4):
+            rid = rng.choice(list(live))
+            toks, pos = live[rid]
+            n = min(len(toks) - pos, rng.choice([1, 2, 5, 9]))
+            if m.can_reserve(rid, pos + n, pos, pos + n):
+                m.reserve(rid, pos + n, pos, pos + n)
+                pos += n
+                m.register_full_pages(rid, toks, pos)
+                live[rid] = (toks, pos)
+            if pos == len(toks) or rng.random() < 0.1:
+                m.release(rid)
+                del live[rid]
+        else:
+            toks = rng.choice(stems)[: rng.randrange(5, 40)] + [rng.randrange(50) for _ in range(rng.randrange(1, 9))]
+            first = rng.choice([2, 5, 9])
+            hits = m.can_admit(toks, first)
+            if hits >= 0:
+                cached = m.admit_with_prefix(i, toks, first)
+                assert cached == hits * page and cached < len(toks)
+                hits_seen += hits
+                for g, table in enumerate(m.requests[i].tables):
+                    lo = m._first_needed_page(g, cached)
+                    assert all(p == -1 for p in table[:min(lo, hits)]) and all(p >= 0 for p in table[lo:hits])
+                live[i] = (toks, m.requests[i].num_tokens)
+                m.register_full_pages(i, toks, cached)
+        m.check()
+    for rid in list(live):
+        m.release(rid)
+    m.check()
+    assert all(pool.num_free == pool.num_pages for pool in m.pools)
+    assert hits_seen > 20
 
 
 # ------------------------------------------------------------------------------ state slots

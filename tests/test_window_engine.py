@@ -2,7 +2,9 @@
 window): LLM.generate under both schedules, with prompts cut into portions of 2, 5 and 16 tokens
 and a window pool so small that pages the window has passed must be given back while prompts are
 still being cut and while requests decode.  The tokens are the plain implementation's; the cache
-manager's books balance afterwards.  Once on the CPU stand-ins of the kernels, once on the GPU."""
+manager's books balance afterwards.  Then with prefix reuse: requests that begin like an earlier one
+leave out the pages that both groups still stand for.  Once on the CPU stand-ins of the kernels,
+once on the GPU."""
 import dataclasses
 
 import pytest
@@ -93,3 +95,58 @@ def test_window_group_through_the_engine(folder, expected, schedule, budget):
     pages = {2: 4, 5: 4, 16: 5}[budget]
     llm = _generate(folder, expected, schedule, budget, pages)
     llm.model.kernels.check_faults()
+
+
+# ------------------------------------------------------------------------------ prefix reuse over both groups
+def _plain_tokens(folder, prompt, n=10):
+    cfg, w = plain.read_folder(folder)
+    ids = list(prompt)
+    for _ in range(n):
+        ids.append(int(torch.argmax(plain.logits(w, cfg, ids, None, order=ORDER, windows=WINDOWS)[-1])))
+    return ids[len(prompt):]
+
+
+def _reuse(folder, window_pages, **where):
+    """One request, then two that begin with its first 43 tokens (five pages and three tokens) and
+    one that does not.  With a window pool that keeps the first request's pages, the two leave out
+    40 tokens each: the all-keys group stands for five pages, the window group for the two that
+    position 40 looks back at (window 12: positions 29..39, pages 3 and 4)."""
+    V = H.CONFIGS["b"]["cfg"].vocab_size
+    stem = H.random_tokens(V, 43, 700)
+    first = stem + H.random_tokens(V, 9, 701)
+    later = [stem + H.random_tokens(V, 14, 702), H.random_tokens(V, 30, 703), stem + H.random_tokens(V, 3, 704)]
+    llm = LLM(folder, dtype="float32", kvcache_block_size=PAGE, num_kvcache_blocks=[40, window_pages],
+              max_num_batched_tokens=16, max_num_seqs=3, **where)
+    cache = llm.runner.cache
+    assert cache.prefix_caching
+    step = llm.step
+
+    def watched_step():
+        out = step()
+        cache.check()
+        return out
+    llm.step = watched_step
+    sp = SamplingParams(temperature=0.0, max_tokens=10)
+    out = llm.generate([first], sp, use_tqdm=False)
+    assert out[0]["token_ids"] == _plain_tokens(folder, first)
+    assert llm.stats["prefill_tokens"] == len(first)
+    outs = llm.generate(later, sp, use_tqdm=False)
+    assert [o["token_ids"] for o in outs] == [_plain_tokens(folder, p) for p in later]
+    assert cache.pools[0].num_free == 40 and cache.pools[1].num_free == window_pages and not cache.requests
+    return llm.stats["prefill_tokens"] - len(first), sum(len(p) for p in later)
+
+
+@pytest.mark.parametrize("window_pages", [12, 5])
+def test_prefix_reuse_with_a_window_group_on_cpu_stand_ins(folder, window_pages):
+    computed, asked = _reuse(folder, window_pages, kernels=TorchKernels(), device="cpu")
+    if window_pages == 12:
+        assert computed == asked - 2 * 40         # both later requests with the stem leave out five pages
+    else:
+        assert computed <= asked                  # the window's pages were taken again: less is left out, or nothing
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window_pages", [12, 5])
+def test_prefix_reuse_with_a_window_group(folder, window_pages):
+    computed, asked = _reuse(folder, window_pages)
+    assert computed == asked - 2 * 40 if window_pages == 12 else computed <= asked
