@@ -4,6 +4,8 @@
 //   q, k:  optional per-head RMS norm over the head (nanovllm/models/qwen3.py:68-70,82-84),
 //          then the rotation of pairs (i, i + rot/2) by the angle table's row of the token's
 //          position (nanovllm/layers/rotary_embedding.py:6-14,44-47), in float, one rounding;
+//          rot, the table's width, is the head size there; a smaller even rot rotates the first
+//          rot channels of the head and leaves the others as they are;
 //          q is written back in place, k in place and into its page slot;
 //   v:     copied into its page slot (nanovllm/layers/attention.py:10-30), stored transposed.
 // Cache layouts: K [pages, kv_heads, page_size, head_dim], V transposed in tiles of keys (common.h).
@@ -40,7 +42,7 @@ __global__ void __launch_bounds__(256)
 qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, PartialInput part, T* q_out, int64_t q_out_stride,
                           int num_q_heads, int num_kv_heads, int head_dim,
                           const void* __restrict__ q_weight, const void* __restrict__ k_weight, int w_is_f32,
-                          float eps, const float* __restrict__ table,
+                          float eps, const float* __restrict__ table, int rot_dim,
                           const int32_t* __restrict__ positions, const int32_t* __restrict__ slots,
                           T* k_cache, T* v_cache, int page_size) {
     const int64_t t = blockIdx.x;
@@ -54,7 +56,12 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, PartialInput part, T* q_ou
     const int row_width = (num_q_heads + 2 * num_kv_heads) * head_dim;
     const int col0 = head * head_dim;
     const int64_t slot = slots ? slots[t] : -1;
-    const int half = head_dim / 2;
+    // A lane holds pairs of channels (a, b): pair i < rot/2 is (i, i + rot/2), which the rotation
+    // turns; the channels from rot on are paired among themselves, (rot + i', rot + i' + rest/2),
+    // and only normed.  With rot = head_dim these are the pairs (i, i + head_dim/2).
+    const int half = head_dim / 2, rot_half = rot_dim / 2, rest_half = (head_dim - rot_dim) / 2;
+#define PAIR_A(i) ((i) < rot_half ? (i) : rot_dim + (i) - rot_half)
+#define PAIR_B(i) ((i) < rot_half ? (i) + rot_half : rot_dim + (i) - rot_half + rest_half)
 
     if (head >= num_q_heads + num_kv_heads) {                       // a v head: copy, transposed
         if (slot < 0 || !v_cache) return;
@@ -76,8 +83,9 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, PartialInput part, T* q_ou
         const int i = lane + j * NVA_WAVE;
         x1[j] = x2[j] = 0.f;
         if (i < half) {
-            x1[j] = part.sums ? partial_value<T>(part, t, row_width, col0 + i) : to_float(row[i]);
-            x2[j] = part.sums ? partial_value<T>(part, t, row_width, col0 + i + half) : to_float(row[i + half]);
+            const int a = PAIR_A(i), b = PAIR_B(i);
+            x1[j] = part.sums ? partial_value<T>(part, t, row_width, col0 + a) : to_float(row[a]);
+            x2[j] = part.sums ? partial_value<T>(part, t, row_width, col0 + b) : to_float(row[b]);
             ss += x1[j] * x1[j] + x2[j] * x2[j];
         }
     }
@@ -88,16 +96,17 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, PartialInput part, T* q_ou
         for (int j = 0; j < NVA_MAX_PER_LANE; ++j) {
             const int i = lane + j * NVA_WAVE;
             if (i < half) {
-                const float w1 = w_is_f32 ? ((const float*)weight)[i] : to_float(((const T*)weight)[i]);
-                const float w2 = w_is_f32 ? ((const float*)weight)[i + half] : to_float(((const T*)weight)[i + half]);
+                const int a = PAIR_A(i), b = PAIR_B(i);
+                const float w1 = w_is_f32 ? ((const float*)weight)[a] : to_float(((const T*)weight)[a]);
+                const float w2 = w_is_f32 ? ((const float*)weight)[b] : to_float(((const T*)weight)[b]);
                 x1[j] = round_through<T>(round_through<T>(x1[j] * scale) * w1);
                 x2[j] = round_through<T>(round_through<T>(x2[j] * scale) * w2);
             }
         }
     }
-    // Rotation of the pair (i, i + head_dim/2), which is exactly (x1, x2).  The table row holds
-    // head_dim/2 cosines, then head_dim/2 sines.
-    const float* angles = table ? table + (int64_t)positions[t] * head_dim : nullptr;
+    // Rotation of the pair (i, i + rot/2), which is exactly (x1, x2).  The table row holds
+    // rot/2 cosines, then rot/2 sines.
+    const float* angles = table ? table + (int64_t)positions[t] * rot_dim : nullptr;
     T* k_dst = nullptr;
     if (!is_q && slot >= 0 && k_cache) {
         const int h = head - num_q_heads;
@@ -108,8 +117,8 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, PartialInput part, T* q_ou
 #pragma unroll
         for (int j = 0; j < NVA_MAX_PER_LANE; ++j) {
             const int i = lane + j * NVA_WAVE;
-            if (i < half) {
-                const float c = angles[i], s = angles[half + i];
+            if (i < rot_half) {
+                const float c = angles[i], s = angles[rot_half + i];
                 const float y1 = x1[j] * c - x2[j] * s;
                 const float y2 = x2[j] * c + x1[j] * s;
                 x1[j] = y1;
@@ -122,20 +131,23 @@ qk_norm_rope_store_kernel(T* qkv, int64_t row_stride, PartialInput part, T* q_ou
         const int i = lane + j * NVA_WAVE;
         if (i < half) {
             const T a = from_float<T>(x1[j]), b = from_float<T>(x2[j]);
+            const int ia = PAIR_A(i), ib = PAIR_B(i);
             if (!part.sums) {
-                row[i] = a;
-                row[i + half] = b;
+                row[ia] = a;
+                row[ib] = b;
             } else if (is_q) {
                 T* qo = q_out + t * q_out_stride + col0;
-                qo[i] = a;
-                qo[i + half] = b;
+                qo[ia] = a;
+                qo[ib] = b;
             }
             if (k_dst) {
-                k_dst[i] = a;
-                k_dst[i + half] = b;
+                k_dst[ia] = a;
+                k_dst[ib] = b;
             }
         }
     }
+#undef PAIR_A
+#undef PAIR_B
 }
 
 // The same work for many tokens at once (portions of prompts).  A workgroup of 256 threads takes
@@ -254,8 +266,9 @@ qk_norm_rope_store_tile_kernel(T* qkv, int64_t row_stride, int tokens, int num_q
 
 static int launch_qk(elem_t* qkv, int64_t row_stride, PartialInput part, elem_t* q_out, int64_t q_out_stride,
                      int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, const void* q_weight,
-                     const void* k_weight, int w_is_f32, float eps, const float* table, const int32_t* positions,
-                     const int32_t* slots, void* k_cache, void* v_cache, int page_size, hipStream_t stream) {
+                     const void* k_weight, int w_is_f32, float eps, const float* table, int rot_dim,
+                     const int32_t* positions, const int32_t* slots, void* k_cache, void* v_cache, int page_size,
+                     hipStream_t stream) {
     if (tokens == 0) return 0;
     if (tokens < 0 || tokens > 0x7fffffff) return nva_fail("qk_norm_rope_store: bad token count %lld", (long long)tokens);
     if (num_q_heads < 0 || num_kv_heads < 0 || num_q_heads + num_kv_heads == 0 || head_dim <= 0)
@@ -266,11 +279,15 @@ static int launch_qk(elem_t* qkv, int64_t row_stride, PartialInput part, elem_t*
     if ((k_cache || v_cache) && (page_size <= 0 || !slots))
         return nva_fail("qk_norm_rope_store: a cache needs a page size and slots");
     if (table && !positions) return nva_fail("qk_norm_rope_store: a rotation table needs positions");
+    if (!table) rot_dim = head_dim;
+    if (rot_dim <= 0 || rot_dim % 2 || rot_dim > head_dim)
+        return nva_fail("qk_norm_rope_store: a rotation of %d channels of a head of %d: it must be even and at most the head",
+                        rot_dim, head_dim);
     const int total = num_q_heads + 2 * num_kv_heads;
     // many tokens of a finished projection: the tiled kernel, where the head size has an instance
     // and the rows can be read in vectors
     const int lph = head_dim / 16;
-    if (!part.sums && tokens >= 64 && head_dim % 16 == 0 && (lph & (lph - 1)) == 0 && lph <= 16 && total <= 65535 &&
+    if (!part.sums && tokens >= 64 && rot_dim == head_dim && head_dim % 16 == 0 && (lph & (lph - 1)) == 0 && lph <= 16 && total <= 65535 &&
         row_stride % 8 == 0 && nva_aligned(qkv, 32) && (!q_weight || nva_aligned(q_weight, 32)) &&
         (!k_weight || nva_aligned(k_weight, 32)) && nva_aligned(table, 32) && nva_aligned(k_cache, 32) &&
         nva_aligned(v_cache, 32)) {
@@ -293,23 +310,24 @@ static int launch_qk(elem_t* qkv, int64_t row_stride, PartialInput part, elem_t*
     const int waves = 4;
     dim3 grid((unsigned)tokens, (total + waves - 1) / waves);
     hipLaunchKernelGGL(qk_norm_rope_store_kernel<elem_t>, grid, dim3(waves * NVA_WAVE), 0, stream, qkv, row_stride, part,
-                       q_out, q_out_stride, num_q_heads, num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table,
+                       q_out, q_out_stride, num_q_heads, num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table, rot_dim,
                        positions, slots, (elem_t*)k_cache, (elem_t*)v_cache, page_size);
     return nva_check_launch("qk_norm_rope_store");
 }
 
 // qkv rows hold [q heads | k heads | v heads] of head_dim each.  q_weight / k_weight may be null
 // (no norm), table may be null (no rotation), the caches may be null (nothing is stored).
-// The kernels read table + positions[t] * head_dim unchecked: the host wrapper takes the largest
+// table rows are rot_dim wide (cosines, then sines), rot_dim even and at most head_dim.
+// The kernels read table + positions[t] * rot_dim unchecked: the host wrapper takes the largest
 // position of the step and refuses one that is not a row of the table.
 NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store)(void* qkv, int64_t row_stride, int64_t tokens, int num_q_heads,
                                                 int num_kv_heads, int head_dim, const void* q_weight,
                                                 const void* k_weight, int w_is_f32, float eps, const float* table,
-                                                const int32_t* positions, const int32_t* slots, void* k_cache,
-                                                void* v_cache, int page_size, hipStream_t stream) {
+                                                int rot_dim, const int32_t* positions, const int32_t* slots,
+                                                void* k_cache, void* v_cache, int page_size, hipStream_t stream) {
     return launch_qk((elem_t*)qkv, row_stride, PartialInput{nullptr, 0, 0, nullptr}, nullptr, 0, tokens, num_q_heads,
-                     num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table, positions, slots, k_cache, v_cache,
-                     page_size, stream);
+                     num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table, rot_dim, positions, slots, k_cache,
+                     v_cache, page_size, stream);
 }
 
 // The same with the packed projection given as float partial sums [splits][tokens][row width]
@@ -317,12 +335,12 @@ NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store)(void* qkv, int64_t row_stride, i
 NVA_EXPORT int NVA_NAME(nva_qk_norm_rope_store_of_partials)(
     const float* sums, int splits, int64_t split_stride, const void* bias, void* q_out, int64_t q_out_stride,
     int64_t tokens, int num_q_heads, int num_kv_heads, int head_dim, const void* q_weight, const void* k_weight,
-    int w_is_f32, float eps, const float* table, const int32_t* positions, const int32_t* slots, void* k_cache,
-    void* v_cache, int page_size, hipStream_t stream) {
+    int w_is_f32, float eps, const float* table, int rot_dim, const int32_t* positions, const int32_t* slots,
+    void* k_cache, void* v_cache, int page_size, hipStream_t stream) {
     if (!sums || splits <= 0 || !q_out) return nva_fail("qk_norm_rope_store_of_partials: no partial sums or no output");
     return launch_qk(nullptr, 0, PartialInput{sums, splits, split_stride, bias}, (elem_t*)q_out, q_out_stride, tokens,
-                     num_q_heads, num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table, positions, slots,
-                     k_cache, v_cache, page_size, stream);
+                     num_q_heads, num_kv_heads, head_dim, q_weight, k_weight, w_is_f32, eps, table, rot_dim, positions,
+                     slots, k_cache, v_cache, page_size, stream);
 }
 
 NVA_DEFINE_LAST_ERROR(nva_rope)

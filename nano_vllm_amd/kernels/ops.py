@@ -87,9 +87,11 @@ def _t(x):
 
 def check_positions_fit(table: torch.Tensor, head_dim: int, max_position: Optional[int]) -> None:
     """The rotary kernels read row positions[t] of the table without a check on the device: a
-    step whose positions are not all rows of the table is refused here."""
-    if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != head_dim or not table.is_contiguous():
-        raise KernelError(f"rotary table must be float32 [positions, {head_dim}]: partial rotation is not built")
+    step whose positions are not all rows of the table is refused here.  The table's width is the
+    number of channels that are rotated: the head's, or fewer (the first of the head)."""
+    if (table.dtype != torch.float32 or table.dim() != 2 or not table.is_contiguous() or table.shape[1] % 2
+            or not 0 < table.shape[1] <= head_dim):
+        raise KernelError(f"rotary table must be float32 [positions, rot], rot even and at most the head's {head_dim}")
     if max_position is None:
         raise KernelError("rotation by a table needs max_position, the bound of the step's positions")
     if max_position > table.shape[0]:
@@ -728,8 +730,8 @@ class HipKernels:
             _i32(slots, tokens, "slots")
         library.call("rope", _suffix(qkv), "nva_qk_norm_rope_store", _p(qkv), c_i64(stride), c_i64(tokens),
                      c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim), _p(q_weight), _p(k_weight), c_i32(wf),
-                     c_f32(eps), _p(table), _p(positions), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size),
-                     self._stream())
+                     c_f32(eps), _p(table), c_i32(0 if table is None else table.shape[1]), _p(positions), _p(slots),
+                     _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
         return qkv[:, : num_heads * head_dim]
 
     def _qk_of_partials(self, qkv: "SplitSum", num_heads, num_kv_heads, head_dim, q_weight, k_weight, eps, table,
@@ -755,8 +757,8 @@ class HipKernels:
         library.call("rope", "bf16", "nva_qk_norm_rope_store_of_partials", _p(qkv.sums), c_i32(qkv.splits),
                      c_i64(tokens * width), _p(qkv.bias), _p(q), c_i64(num_heads * head_dim), c_i64(tokens),
                      c_i32(num_heads), c_i32(num_kv_heads), c_i32(head_dim), _p(q_weight), _p(k_weight), c_i32(wf),
-                     c_f32(eps), _p(table), _p(positions), _p(slots), _p(k_cache), _p(v_cache), c_i32(page_size),
-                     self._stream())
+                     c_f32(eps), _p(table), c_i32(0 if table is None else table.shape[1]), _p(positions), _p(slots),
+                     _p(k_cache), _p(v_cache), c_i32(page_size), self._stream())
         return q
 
     @staticmethod

@@ -51,8 +51,10 @@ def test_positions_must_be_rows_of_the_rotary_table():
         check_positions_fit(table, 16, 129)
     with pytest.raises(KernelError, match="needs max_position"):
         check_positions_fit(table, 16, None)
-    with pytest.raises(KernelError, match="float32"):
-        check_positions_fit(table, 32, 10)
+    check_positions_fit(table, 32, 10)                  # a table narrower than the head: the first 16 channels are rotated
+    for head_dim, bad in ((8, table), (16, torch.zeros((128, 7))), (16, torch.zeros((128, 16), dtype=torch.float64))):
+        with pytest.raises(KernelError, match="float32"):
+            check_positions_fit(bad, head_dim, 10)
 
 
 def test_row_counts_choose_the_product_kernel():

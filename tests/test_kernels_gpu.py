@@ -560,6 +560,51 @@ def test_qk_norm_rope_store_of_a_long_portion(hip, ref, dtype, hq, hkv, D, page)
     assert torch.equal(a[:, (hq + hkv) * D:], qkv[:, (hq + hkv) * D:])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hq,hkv,D,rot,page,T", [(4, 2, 16, 8, 4, 37), (5, 5, 48, 16, 16, 37), (8, 2, 128, 64, 256, 100),
+                                                  (3, 1, 80, 30, 64, 70), (2, 2, 256, 2, 32, 9), (7, 1, 64, 62, 8, 37)])
+def test_qk_norm_rope_store_with_a_rotation_of_fewer_channels(hip, ref, dtype, hq, hkv, D, rot, page, T):
+    """A table narrower than the head: the first `rot` channels are rotated in pairs (i, i + rot/2)
+    by the angles of a head of that size, the others are only normed.  Checked against the stand-in
+    and, channel by channel, against the plain rotation of the slice."""
+    pages = (T + page - 1) // page + 2
+    k = hip[dtype]
+    qkv = _rand((T, (hq + 2 * hkv) * D), dtype, 51)
+    qw, kw = _rand((D,), dtype, 52) + 1, _rand((D,), dtype, 53) + 1
+    table = ref.rotary_table(_inv_freq(rot, 1e4), 500)
+    assert table.shape == (500, rot)
+    positions = torch.randint(0, 500, (T,), dtype=torch.int32, device=DEV)
+    slots = torch.randperm(pages * page)[:T].to(torch.int32).to(DEV)
+    caches = [new_caches(pages, hkv, D, page, dtype, DEV) for _ in range(2)]
+    a, b = qkv.clone(), qkv.clone()
+    qa = k.qk_norm_rope_store(a, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[0], max_position=500)
+    qb = ref.qk_norm_rope_store(b, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches[1], max_position=500)
+    _close(qa, qb, dtype, "q")
+    _close(a, b, dtype, "k in place")
+    _close(caches[0][0], caches[1][0], dtype, "k cache")
+    assert torch.equal(caches[0][1], caches[1][1])
+    # without norm weights: the channels from rot on come back as they were, and the first rot are
+    # the plain rotation of that slice
+    c = qkv.clone()
+    qc = k.qk_norm_rope_store(c, hq, hkv, D, None, None, 1e-6, table, positions, None, None, None, max_position=500)
+    heads = qkv[:, : hq * D].reshape(T, hq, D)
+    got = qc.reshape(T, hq, D)
+    assert torch.equal(got[..., rot:], heads[..., rot:])
+    ang = plain.rope_angles(rot, positions.cpu(), 1e4)
+    want = plain.apply_rope(heads[..., :rot].float().cpu(), ang)
+    _close(got[..., :rot].cpu(), want.to(dtype), dtype, "rotated slice")
+    # partial sums take the same kernel
+    if dtype == torch.bfloat16:
+        from nano_vllm_amd.kernels.ops import SplitSum
+        width = (hq + 2 * hkv) * D
+        sums = torch.stack([qkv.float() * 0.75, qkv.float() * 0.25])
+        part = SplitSum(k, sums.reshape(-1), 2, T, width, None)
+        assert torch.equal(part.tensor(), qkv)
+        caches2 = new_caches(pages, hkv, D, page, dtype, DEV)
+        qp = k.qk_norm_rope_store(part, hq, hkv, D, qw, kw, 1e-6, table, positions, slots, *caches2, max_position=500)
+        assert torch.equal(qp, qa) and torch.equal(caches2[0], caches[0][0]) and torch.equal(caches2[1], caches[0][1])
+
+
 def test_qk_refusals(hip):
     from nano_vllm_amd.kernels import KernelError
     k = hip[torch.float32]
@@ -567,6 +612,11 @@ def test_qk_refusals(hip):
         k.qk_norm_rope_store(torch.zeros((2, 100), device=DEV), 2, 1, 16, None, None, 1e-6, None, None, None, None, None)
     with pytest.raises(KernelError, match="head_dim"):
         k.qk_norm_rope_store(torch.zeros((2, 4 * 1024), device=DEV), 2, 1, 1024, None, None, 1e-6, None, None, None, None, None)
+    positions = torch.zeros(2, dtype=torch.int32, device=DEV)
+    for width in (18, 7):                                          # wider than the head; odd
+        with pytest.raises(KernelError, match="rot even and at most"):
+            k.qk_norm_rope_store(torch.zeros((2, 4 * 16), device=DEV), 2, 1, 16, None, None, 1e-6,
+                                 torch.zeros((10, width), device=DEV), positions, None, None, None, max_position=1)
 
 
 # ------------------------------------------------------------------------------ attention

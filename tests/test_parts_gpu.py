@@ -60,6 +60,17 @@ def test_position_encoding_part():
     assert float((t[:, :24] - ang.cos()).abs().max()) < 2e-6 and float((t[:, 24:] - ang.sin()).abs().max()) < 2e-6
     none = make_part("position_encoding", PartSpec("none"), _ctx(torch.float32))
     assert none.rotary_table() is None
+    # fewer rotated channels than the head has: a narrower table, with the angles of a head of that size
+    part = make_part("position_encoding", PartSpec("rotary_neox", {"head_dim": 48, "rotary_dim": 20, "theta": 5e5,
+                                                                   "max_position": 300}), _ctx(torch.float32))
+    t = part.rotary_table().cpu()
+    ang = plain.rope_angles(20, torch.arange(300), 5e5)
+    assert t.shape == (300, 20)
+    assert float((t[:, :10] - ang.cos()).abs().max()) < 2e-6 and float((t[:, 10:] - ang.sin()).abs().max()) < 2e-6
+    for bad in (0, 21, 50):
+        with pytest.raises(ValueError, match="rotated channels"):
+            make_part("position_encoding", PartSpec("rotary_neox", {"head_dim": 48, "rotary_dim": bad, "theta": 5e5}),
+                      _ctx(torch.float32))
 
 
 @pytest.mark.parametrize("dt", ["float32", "bfloat16"])
@@ -125,6 +136,63 @@ def test_attention_part_in_portions(dt, window):
     assert _err(torch.cat(got), want) < TOL[dt]
     if window:
         assert cache.table("r", 0)[0] == -1                  # the window has passed the first pages
+    part.kernels.check_faults()
+
+
+@pytest.mark.parametrize("dt", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rot", [12, 32])
+def test_attention_part_with_a_rotation_of_fewer_channels(dt, rot):
+    """The attention part with a position encoding that rotates the first `rot` of 32 channels,
+    through the fused kernel, in portions and single tokens, against a computation in double on
+    the whole sequence.  rot = 32 is the package's ordinary case, by the same computation."""
+    dtype = DTYPES[dt]
+    heads, kv_heads, D, hidden, T = 6, 3, 32, 96, 90
+    ctx = _ctx(dtype, hidden)
+    ctx.position_encodings["rope"] = make_part("position_encoding", PartSpec(
+        "rotary_neox", {"head_dim": D, "rotary_dim": rot, "theta": 1e4, "max_position": 256}), ctx)
+    part = make_part("mixer", PartSpec("attention", {
+        "hidden_size": hidden, "num_heads": heads, "num_kv_heads": kv_heads, "head_dim": D, "qk_norm": True,
+        "eps": 1e-6, "position_encoding": "rope", "window": None}), ctx)
+    w = {"q": _rand((heads * D, hidden), 1, 0.2), "k": _rand((kv_heads * D, hidden), 2, 0.2),
+         "v": _rand((kv_heads * D, hidden), 3, 0.2), "o": _rand((hidden, heads * D), 4, 0.2),
+         "qn": 1 + _rand((D,), 5, 0.1), "kn": 1 + _rand((D,), 6, 0.1)}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    part.weights["qkv_proj.weight"] = torch.cat([w["q"], w["k"], w["v"]]).to(DEV)
+    part.weights["o_proj.weight"] = w["o"].to(DEV)
+    part.weights["q_norm.weight"], part.weights["k_norm.weight"] = w["qn"].to(DEV), w["kn"].to(DEV)
+    x = _rand((T, hidden), 9).to(dtype)
+
+    f = {k: v.double() for k, v in w.items()}
+    xd = x.double()
+    norm = lambda v, g: v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + 1e-6) * g
+    ang = torch.arange(T, dtype=torch.float64)[:, None] / (1e4 ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot))[None, :]
+    c, s_ = ang.cos()[:, None, :], ang.sin()[:, None, :]
+
+    def rotate(v):                                                  # [T, heads, D]: pairs (i, i + rot/2) of the first rot
+        a, b = v[..., : rot // 2], v[..., rot // 2: rot]
+        return torch.cat((a * c - b * s_, b * c + a * s_, v[..., rot:]), dim=-1)
+
+    q = rotate(norm((xd @ f["q"].T).reshape(T, heads, D), f["qn"]))
+    k = rotate(norm((xd @ f["k"].T).reshape(T, kv_heads, D), f["kn"])).repeat_interleave(heads // kv_heads, 1)
+    v = (xd @ f["v"].T).reshape(T, kv_heads, D).repeat_interleave(heads // kv_heads, 1)
+    sc = torch.einsum("thd,shd->hts", q, k) * D ** -0.5
+    sc = sc.masked_fill(torch.ones(T, T).triu(1).bool(), float("-inf"))
+    want = (torch.einsum("hts,shd->thd", torch.softmax(sc, -1), v).reshape(T, heads * D) @ f["o"].T).float()
+
+    need = part.cache_need()
+    cache = CacheManager([CacheGroup(None, (0,))], 8, 14, enable_prefix_caching=False)
+    from torch_kernels import new_caches
+    kc, vc = new_caches(14, need.num_kv_heads, need.head_dim, 8, dtype, DEV)
+    lc = LayerCache(group=0, k=kc, v=vc)
+    cache.admit("r")
+    got, pos = [], 0
+    for n in (13, 1, 1, 66, 2, 7):                                  # 66: as many tokens as take the tiled kernel where it serves
+        cache.reserve("r", pos + n, first_query=pos)
+        batch = build_batch([StepEntry("r", [0] * n, pos, [])], cache, 8, 10, DEV)
+        y = part.forward(x[pos:pos + n].to(DEV), batch, lc)
+        got.append(y.tensor() if hasattr(y, "tensor") else y)
+        pos += n
+    assert _err(torch.cat(got), want) < (1e-5 if dt == "float32" else 2.0 ** -5)
     part.kernels.check_faults()
 
 

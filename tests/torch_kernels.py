@@ -115,10 +115,11 @@ class TorchKernels:
                 x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
                 x = _round(_round(x, dt) * w.float(), dt)
             if table is not None:
-                row = table[positions.long()]                       # [T, D]
-                cos, sin = row[:, None, : D // 2], row[:, None, D // 2:]
-                x1, x2 = x[..., : D // 2], x[..., D // 2:]
-                x = torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), dim=-1)
+                row = table[positions.long()]                       # [T, R]: the first R channels of a head are rotated
+                R = row.shape[1]
+                cos, sin = row[:, None, : R // 2], row[:, None, R // 2:]
+                x1, x2 = x[..., : R // 2], x[..., R // 2:R]
+                x = torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin, x[..., R:]), dim=-1)
             return x.to(dt)
 
         q = prepare(qkv[:, :qd], num_heads, q_weight)
