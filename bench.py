@@ -35,7 +35,7 @@ def parse_args():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
-    ap.add_argument("--shape", default="qwen3-8b", help="a named shape of nano_vllm_amd.models.shapes (qwen3-8b, qwen3-14b, qwen3-32b)")
+    ap.add_argument("--shape", default="qwen3-8b", help="a named shape of nano_vllm_amd.models.shapes (qwen3-0.6b ... qwen3-32b)")
     ap.add_argument("--layers", type=int, default=None, help="layers to build (default: all the shape has)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--page-size", type=int, default=256)

@@ -147,7 +147,7 @@ def main(argv=None) -> int:
     t.set_defaults(fn=cmd_throughput)
     r = sub.add_parser("random-model", help="write a model folder with seeded random weights")
     r.add_argument("--config", default=None, help="a config.json of the architecture")
-    r.add_argument("--shape", default=None, help="a named shape instead: tiny-a, tiny-b, qwen3-8b, qwen3-14b, qwen3-32b")
+    r.add_argument("--shape", default=None, help="a named shape instead: tiny-a, tiny-b, qwen3-0.6b, qwen3-1.7b, qwen3-4b, qwen3-8b, qwen3-14b, qwen3-32b")
     r.add_argument("--config-only", action="store_true", help="write config.json only (for --random-weights)")
     r.add_argument("--seed", type=int, default=0)
     r.add_argument("--out", required=True)
