@@ -103,9 +103,10 @@ def real_size_folder(tmp_path_factory):
 
 # 8B: 32 heads in groups of four; 14B: 40 heads in groups of five, widths of 5120 and 17408;
 # 32B: 64 heads in groups of eight, 25600 inner channels: other instances of the product and
-# attention kernels than the 8B sizes run
+# attention kernels than the 8B sizes run.  0.6B, 1.7B, 4B: groups of two, q heads wider than the
+# model (2048 of 1024), widths of 2560 and 9728, a tied head.
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["qwen3-8b", "qwen3-14b", "qwen3-32b"])
+@pytest.mark.parametrize("name", ["qwen3-0.6b", "qwen3-1.7b", "qwen3-4b", "qwen3-8b", "qwen3-14b", "qwen3-32b"])
 def test_layer_sizes_of_the_named_shapes(real_size_folder, name, dtype):
     """Two layers with the layer sizes of the benchmarks' shapes: float32 against the plain
     implementation, whole, decoded and in portions; bfloat16 against the plain implementation with
