@@ -84,6 +84,13 @@ class Model:
         if getattr(self.head, "tied", False):
             self.head.weights["weight"] = self.embedding.weights["weight"]
 
+        def told(part: Part) -> None:
+            for child in part.children().values():
+                told(child)
+            part.on_weights_loaded()
+        for part in [*self.position_encodings.values(), self.embedding, *self.blocks, self.final_norm, self.head]:
+            told(part)
+
     def num_parameters(self) -> int:
         return sum(int(torch.tensor(d.shape).prod()) for _, _, d in self.param_table.values())
 

@@ -314,8 +314,15 @@ def test_another_embedding_and_head_are_registered_not_edited_in(tmp_path):
     scale, cap = 3.0, 0.05
 
     class ScaledEmbedding(TokenEmbedding):
+        told = 0
+
+        def on_weights_loaded(self):                  # called once, after every parameter is there
+            assert self.weights["weight"].shape == (384, 96)
+            type(self).told += 1
+            self.factor = torch.tensor(float(self.params["scale"]))
+
         def forward(self, ids):
-            return super().forward(ids) * float(self.params["scale"])
+            return super().forward(ids) * self.factor
 
     class CappedHead(OutputHead):
         def forward(self, x):
@@ -357,6 +364,7 @@ def test_another_embedding_and_head_are_registered_not_edited_in(tmp_path):
         r = H.make_runner(folder, "float32", 8, 16, device="cpu", kernels=TorchKernels())
         runs[name] = H.run_portions(r, "x", toks, [25, 1, 14])
     want = torch.tanh(runs["scaled"] / cap) * cap
+    assert ScaledEmbedding.told == 1
     assert H.rel_err(runs["toy"], want) < TOL
     assert H.rel_err(runs["base"], runs["scaled"]) > 1e-2        # the scale moves the logits: the check above can fail
     assert (runs["scaled"].abs() > cap).any()                    # and so does the cap
