@@ -81,8 +81,30 @@ class SplitSum:
         return self._tensor
 
 
+class PendingProduct:
+    """A bfloat16 product of many rows that the library has not run yet: x and the weight.  The
+    norm that adds it to the residual stream runs it as residual <- residual + x @ weight.T, the sum
+    in the product's own epilogue (float, rounded once), which saves a pass over the product;
+    anything else gets `tensor()`, the plain product."""
+
+    def __init__(self, x: torch.Tensor, weight: torch.Tensor):
+        self.x, self.weight = x, weight
+        self.dtype = x.dtype
+        self.device = x.device
+        self.shape = (x.shape[0], weight.shape[0])
+        self._tensor = None
+
+    def tensor(self) -> torch.Tensor:
+        if self._tensor is None:
+            self._tensor = torch.nn.functional.linear(self.x, self.weight)
+        return self._tensor
+
+    def add_to(self, residual: torch.Tensor) -> torch.Tensor:
+        return residual.addmm_(self.x, self.weight.t())
+
+
 def _t(x):
-    return x.tensor() if isinstance(x, SplitSum) else x
+    return x.tensor() if isinstance(x, (SplitSum, PendingProduct)) else x
 
 
 def check_positions_fit(table: torch.Tensor, head_dim: int, max_position: Optional[int]) -> None:
@@ -297,6 +319,7 @@ class HipKernels:
     def rms_norm(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None):
         if isinstance(x, SplitSum):
             return self._norm_of_partials(x, None, weight, eps, out)
+        x = _t(x)
         rows, width, xs = _rows2d(x, "rms_norm input")
         wf = self._norm_weight(weight, width, x)
         if out is None:
@@ -313,6 +336,11 @@ class HipKernels:
         """residual <- x + residual (in place); returns (norm(residual) * weight, residual)."""
         if isinstance(x, SplitSum):
             return self._norm_of_partials(x, residual, weight, eps, out), residual
+        if isinstance(x, PendingProduct):
+            if (residual.dim() != 2 or tuple(residual.shape) != x.shape or residual.dtype != x.dtype
+                    or residual.stride(1) != 1):
+                raise KernelError("add_rms_norm: residual does not match the input")
+            return self.rms_norm(x.add_to(residual), weight, eps, out=out), residual
         rows, width, xs = _rows2d(x, "add_rms_norm input")
         rrows, rw, rs = _rows2d(residual, "add_rms_norm residual")
         if (rrows, rw) != (rows, width) or residual.dtype != x.dtype:
@@ -349,7 +377,8 @@ class HipKernels:
         """y = x @ weight.T (+ bias), weight [out, in].  float32 inputs run the engine's own
         float kernel; bfloat16 inputs with many rows run the library product (also for a float
         result of more than 16 rows), with few rows the weight-streaming kernels.  deferred: the caller hands the result to a norm or to the q/k
-        preparation only, so a product split over k may come back as a SplitSum."""
+        preparation only, so a product split over k may come back as a SplitSum, and a library
+        product as a PendingProduct."""
         x = _t(x)
         m, k, xs = _rows2d(x, "linear input")
         n, wk, ws = _rows2d(weight, "linear weight")
@@ -402,6 +431,8 @@ class HipKernels:
                     self._linear_skinny(x[r0:r1], xs, weight, ws, bias, out[r0:r1], os_, out_float32, False, r1 - r0, n, k)
                 return out
         if x.dtype == torch.bfloat16 and not out_float32:
+            if deferred and bias is None and out is None and self.fuse_split_sums and xs == k and ws == k:
+                return PendingProduct(x, weight)        # the library's product, run by whoever takes it
             y = torch.nn.functional.linear(x, weight, bias)
             if out is not None:
                 out.copy_(y)
@@ -710,6 +741,7 @@ class HipKernels:
         if isinstance(qkv, SplitSum):
             return self._qk_of_partials(qkv, num_heads, num_kv_heads, head_dim, q_weight, k_weight, eps, table,
                                         positions, slots, k_cache, v_cache)
+        qkv = _t(qkv)
         tokens, width, stride = _rows2d(qkv, "qkv")
         if width != (num_heads + 2 * num_kv_heads) * head_dim:
             raise KernelError(f"qkv width {width} is not (heads + 2*kv_heads) * head_dim = "

@@ -484,6 +484,38 @@ def test_split_products_are_consumed_by_norm_and_qk_kernels(hip, ref):
     assert torch.equal(k.rms_norm(y, nw, 1e-6), k.rms_norm(done, nw, 1e-6))
 
 
+def test_library_products_are_run_by_the_norm_that_adds_them(hip):
+    """A product of many rows handed to the residual norm is run there, the sum in the product's
+    epilogue: residual + x W^T in float rounded once, then the norm of that; every other
+    consumer gets the plain product."""
+    from nano_vllm_amd.kernels.ops import PendingProduct
+    k = hip[torch.bfloat16]
+    m, kk, n = 300, 1024, 768
+    x = _rand((m, kk), torch.bfloat16, 40)
+    w = _rand((n, kk), torch.bfloat16, 41, 0.05)
+    res = _rand((m, n), torch.bfloat16, 42)
+    nw = _rand((n,), torch.bfloat16, 43) + 1
+    y = k.linear(x, w, deferred=True)
+    assert isinstance(y, PendingProduct) and y.shape == (m, n)
+    assert torch.equal(y.tensor(), k.linear(x, w))
+    assert torch.equal(k.rms_norm(y, nw, 1e-6), k.rms_norm(k.linear(x, w), nw, 1e-6))
+    r = res.clone()
+    a, r_out = k.add_rms_norm(k.linear(x, w, deferred=True), r, nw, 1e-6)
+    assert r_out is r
+    want_r = x.double() @ w.double().t() + res.double()
+    _close(r, want_r, torch.bfloat16, "residual + product")
+    assert torch.equal(a, k.rms_norm(r, nw, 1e-6))
+    # the sum is rounded once: closer to the exact sum than product and sum rounded in turn
+    two = (k.linear(x, w).float() + res.float()).bfloat16()
+    assert float((r.double() - want_r).abs().mean()) <= float((two.double() - want_r).abs().mean())
+    # with a bias, or a result that is asked for as a tensor, nothing is left pending
+    bias = _rand((n,), torch.bfloat16, 44)
+    assert isinstance(k.linear(x, w, bias, deferred=True), torch.Tensor)
+    assert isinstance(k.linear(x, w), torch.Tensor)
+    with pytest.raises(Exception, match="residual does not match"):
+        k.add_rms_norm(k.linear(x, w, deferred=True), res[:10].clone(), nw, 1e-6)
+
+
 # ------------------------------------------------------------------------------ rotation and cache write
 def _inv_freq(D, theta):
     return (1.0 / (theta ** (torch.arange(0, D, 2, dtype=torch.float) / D))).to(DEV)
