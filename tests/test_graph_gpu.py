@@ -143,3 +143,48 @@ def test_graphs_captured_at_start_give_the_eager_steps():
     small.enable_decode_graphs(max_batch=8, max_len=c["cfg"].max_position_embeddings)
     assert small.capture_decode_graphs() == 3 and sorted(small._graphs) == [1, 2, 4]
     graphed.kernels.check_faults()
+
+
+def test_a_captured_step_of_more_rows_than_the_engines_own_products_take():
+    """More than 256 single tokens: the products are the library's, the residual sum runs in their
+    epilogue, the logits come from the library's product with a float result, all inside the
+    captured step.  Every replay against the eager step, eager work between the replays."""
+    name, dtype, n = "b", "bfloat16", 272
+    c = H.CONFIGS[name]
+    folder = H.model_folder(name, dtype)
+    eager = H.make_runner(folder, dtype, c["page"], 2 * n + 8, max_requests=n + 1)
+    graphed = H.make_runner(folder, dtype, c["page"], 2 * n + 8, max_requests=n + 1)
+    graphed.enable_decode_graphs(max_batch=n, max_len=c["cfg"].max_position_embeddings)
+    V = c["cfg"].vocab_size
+    reqs = {f"r{i}": H.random_tokens(V, 3 + i % 5 + 6, 300 + i) for i in range(n)}
+    extra = H.random_tokens(V, 37, 99)
+    pos = {}
+    for r in (eager, graphed):
+        for rid, toks in reqs.items():
+            r.cache.admit(rid)
+            r.cache.reserve(rid, len(toks) - 6)
+        r.step([StepEntry(rid, toks[:-6], 0, []) for rid, toks in reqs.items()])
+    for rid, toks in reqs.items():
+        pos[rid] = len(toks) - 6
+    for step in range(5):
+        outs = []
+        for r in (eager, graphed):
+            entries = []
+            for rid in reqs:
+                r.cache.reserve(rid, pos[rid] + 1)
+                entries.append(StepEntry(rid, [reqs[rid][pos[rid]]], pos[rid], [0]))
+            outs.append(r.step(entries).clone())
+            if step % 2 == 1:
+                r.cache.admit("x")
+                r.cache.reserve("x", len(extra))
+                r.step([StepEntry("x", extra, 0, [len(extra) - 1])])
+                r.cache.release("x")
+            torch.cuda.synchronize()
+        for rid in reqs:
+            pos[rid] += 1
+        assert H.rel_err(outs[1], outs[0]) < 1e-5, f"replay {step} differs from the eager step"
+    assert sorted(graphed._graphs) == [n]
+    rid = "r7"
+    want = H.plain_logits(folder, reqs[rid][:pos[rid]], "bfloat16")
+    assert H.rel_err(outs[1][7].cpu(), want[-1]) < 2e-2
+    graphed.kernels.check_faults()
