@@ -9,7 +9,13 @@
 // request's draw does not depend on what else is in the batch:
 //   bits = mix64(key ^ entry);  u = ((bits >> 40) + 0.5) / 2^24;  E = -log(u)
 // with mix64 the splitmix64 finaliser; the key is made on the host from (seed, request,
-// position).  Noise and scores are computed in double.
+// position).  Noise and scores are computed in double.  Two logarithms in double for every entry
+// are most of that work, and only the largest score matters: a workgroup first takes all scores of
+// its chunk in float, with the fast logarithm, keeps them in registers and finds their maximum; then only
+// the entries whose float score lies within SAMPLE_WINDOW of that maximum (a few), and those whose u
+// lies in the far tails, where the float score is poor, are taken in double.  The float score is off
+// by a few thousandths at most (below), the window is a hundred times that, so the entry with the
+// largest score in double is always among them, and it is the one chosen.
 #include "common.h"
 
 __device__ __forceinline__ uint64_t mix64(uint64_t z) {
@@ -21,6 +27,8 @@ __device__ __forceinline__ uint64_t mix64(uint64_t z) {
 
 #define SAMPLE_THREADS 256
 #define SAMPLE_CHUNK 8192         // entries of a row per workgroup
+#define SAMPLE_WINDOW 0.5f        // float scores this far below the largest are still taken in double
+#define SAMPLE_TAIL 1024u         // u below SAMPLE_TAIL / 2^24 or above 1 - SAMPLE_TAIL / 2^24: always in double
 
 __device__ __forceinline__ bool better(double s, int i, double best, int best_idx) {
     // a NaN score never wins (its index stays 0x7fffffff); the lowest index wins a tie
@@ -35,6 +43,17 @@ __device__ __forceinline__ double score(float logit, float temp, uint64_t key, i
         s = s / (double)temp - log(-log(u));
     }
     return s;
+}
+
+// The score in float, or +inf for an entry that is to be taken in double whatever the others' scores.
+// Between the tails |d log(-log u) / du| is at most 2^24 / SAMPLE_TAIL, the float u is off by 2^-25
+// (it has no bit for the half) and the fast logarithm by a few units in the last place, also of the
+// small -log u near u = 1: together under 2e-3; the quotient logit / T adds 2e-7 of itself.
+__device__ __forceinline__ float float_score(float logit, float inv_temp, uint64_t key, int entry) {
+    const uint32_t k24 = (uint32_t)(mix64(key ^ (uint64_t)entry) >> 40);
+    if (k24 < SAMPLE_TAIL || k24 >= (1u << 24) - SAMPLE_TAIL) return INFINITY;
+    const float u = ((float)k24 + 0.5f) * (1.f / 16777216.f);
+    return logit * inv_temp - __logf(-__logf(u));
 }
 
 // The best entry of a block's threads: within the waves, then across them (thread 0 holds it).
@@ -79,6 +98,50 @@ sample_chunk_kernel(const float* __restrict__ logits, int64_t row_stride, int vo
     int best_idx = 0x7fffffff;
     const bool vec = (row_stride % 4 == 0) && ((uintptr_t)logits % 16 == 0);
     const int vec_end = vec ? begin + ((end - begin) & ~3) : begin;
+    if (temp > 0.f) {
+        // ---- every score in float, kept in registers (a thread walks SAMPLE_CHUNK / SAMPLE_THREADS
+        // entries); their maximum over the chunk (the tails and NaN aside)
+        constexpr int PER = SAMPLE_CHUNK / SAMPLE_THREADS;
+        __shared__ float max_s[SAMPLE_THREADS / NVA_WAVE];
+        const float inv_temp = 1.f / temp;
+        // entry j of this thread: four in a row per turn where rows can be read in vectors
+        auto entry = [&](int j) { return vec ? begin + (j / 4) * (SAMPLE_THREADS * 4) + threadIdx.x * 4 + j % 4
+                                             : begin + j * SAMPLE_THREADS + threadIdx.x; };
+        float f[PER], top = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < PER; j += 4) {
+            float v[4];
+            if (vec && entry(j) + 3 < end) {
+                const float4 v4 = *reinterpret_cast<const float4*>(l + entry(j));
+                v[0] = v4.x; v[1] = v4.y; v[2] = v4.z; v[3] = v4.w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = entry(j + e) < end ? l[entry(j + e)] : 0.f;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                f[j + e] = entry(j + e) < end ? float_score(v[e], inv_temp, key, entry(j + e)) : -INFINITY;
+                if (f[j + e] < INFINITY) top = fmaxf(top, f[j + e]);      // not for a NaN either
+            }
+        }
+        top = wave_max(top);
+        if (threadIdx.x % NVA_WAVE == 0) max_s[threadIdx.x / NVA_WAVE] = top;
+        __syncthreads();
+        top = max_s[0];
+#pragma unroll
+        for (int w = 1; w < SAMPLE_THREADS / NVA_WAVE; ++w) top = fmaxf(top, max_s[w]);
+        // ---- in double: what may be the largest.  (No finite float score at all: everything.)
+        const float least = top - (SAMPLE_WINDOW + 4e-6f * fabsf(top));
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            if (f[j] < least || entry(j) >= end) continue;        // the comparison is false for +inf and for a NaN
+            const double s = score(l[entry(j)], temp, key, entry(j));
+            if (s == s && better(s, entry(j), best, best_idx)) {
+                best = s;
+                best_idx = entry(j);
+            }
+        }
+    } else {
     for (int i = begin + threadIdx.x * 4; i < vec_end; i += SAMPLE_THREADS * 4) {
         const float4 v4 = *reinterpret_cast<const float4*>(l + i);
         const float v[4] = {v4.x, v4.y, v4.z, v4.w};
@@ -97,6 +160,7 @@ sample_chunk_kernel(const float* __restrict__ logits, int64_t row_stride, int vo
             best = s;
             best_idx = i;
         }
+    }
     }
     block_best(best, best_idx);
     if (threadIdx.x == 0) {

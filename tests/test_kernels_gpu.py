@@ -1046,6 +1046,50 @@ def test_sampling_matches_the_plain_draw(hip):
     assert got == want and got[0] == 17
 
 
+def _exact_draws(logits, temps, keys):
+    """argmax(l / T - log(-log u)) in double for whole rows at once: the kernel's generator written with
+    torch's 64-bit integers (multiplication wraps; the shifts are made logical by masking)."""
+    def shr(z, n):
+        return (z >> n) & ((1 << (64 - n)) - 1)
+
+    def as_i64(c):
+        return c - (1 << 64) if c >= (1 << 63) else c
+    rows, vocab = logits.shape
+    entry = torch.arange(vocab, dtype=torch.int64, device=logits.device)
+    out = []
+    for r in range(rows):
+        z = (keys[r] ^ entry) + as_i64(0x9E3779B97F4A7C15)
+        z = (z ^ shr(z, 30)) * as_i64(0xBF58476D1CE4E5B9)
+        z = (z ^ shr(z, 27)) * as_i64(0x94D049BB133111EB)
+        z = z ^ shr(z, 31)
+        u = (shr(z, 40).double() + 0.5) / 16777216.0
+        score = logits[r].double()
+        if float(temps[r]) > 0:
+            score = score / float(temps[r]) - torch.log(-torch.log(u))
+        out.append(int(torch.argmax(score)))
+    return out
+
+
+def test_sampling_passes_by_no_entry_that_wins(hip):
+    """The kernel takes the score of most entries in float first and passes them by when they cannot
+    beat the best so far; the entry it chooses is the one the scores in double choose: rows of the
+    size of a real vocabulary, temperatures from 0.01 to 50, logits that are large, flat, or equal."""
+    from nano_vllm_amd.sampling.sampler import noise_key
+    k = hip[torch.float32]
+    V, R = 151936, 48
+    logits = _rand((R, V), torch.float32, 61, 3.0)
+    logits[8:16] *= 20.0                                            # large
+    logits[16:24] *= 1e-3                                           # flat: the noise decides
+    logits[24:28] = 1.5                                             # all equal
+    logits[28:32] = -80.0 + _rand((4, V), torch.float32, 62, 1e-2)
+    temps = torch.tensor([[0.01, 0.1, 0.6, 1.0, 2.0, 7.0, 50.0, 0.3][r % 8] for r in range(R)], device=DEV)
+    keys = torch.tensor([noise_key(5, r, 1000 + 17 * r) for r in range(R)], dtype=torch.int64, device=DEV)
+    assert _exact_draws(logits[:3, :1001], temps[:3], keys[:3]) == \
+        [plain.sample(logits[r, :1001].cpu(), float(temps[r]), seed=5, request=r, position=1000 + 17 * r) for r in range(3)]
+    got = k.sample(logits, temps, keys).tolist()
+    assert got == _exact_draws(logits, temps, keys)
+
+
 def test_sampling_over_a_vocabulary_of_several_chunks(hip):
     """A row is cut into chunks of 8192 entries for the first pass: ties across chunks, a maximum
     at a chunk's edge, rows of a wider tensor (a stride that is no multiple of four), NaN entries."""
