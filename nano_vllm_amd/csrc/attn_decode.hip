@@ -80,7 +80,8 @@ __device__ __forceinline__ void load_chunk(int base, bf16x8* ka, bf16x8* kb, bf1
 // Every wave gets the same amount of work, whatever the lengths of the requests: the chunks (32
 // keys) that the tokens see are counted through, token after token, and cut into quotas of equal
 // size, one quota for each of the W waves that work on a kv head (W = waves of the launch / kv
-// heads, as many as the GPU holds at once); at least two chunks a quota, and at most what 62 pages
+// heads, as many as the GPU holds at once); at least two chunks a quota (four for a few long
+// requests, see nva_attn_decode_plan_size), and at most what 62 pages
 // hold (a wave keeps the block table entries of what it reads in one register per lane), in which
 // case a wave takes several quotas in turn.  A quota is one or more segments: (token, keys lo..hi).
 // A token cut by a quota's edge has several segments, which a second kernel merges; a token with
