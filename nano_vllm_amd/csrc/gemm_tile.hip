@@ -37,6 +37,7 @@ struct TileArgs {
     const __bf16* w; int64_t w_stride; const __bf16* bias;
     void* y; int64_t y_stride; float* partial; int mode;
     int M, N, K, chunks_per_range;
+    int cols_per_wg;        // columns of y a workgroup takes: those of its tile, or fewer (the tile's other rows of W are not fetched)
 };
 
 // 16 bytes per lane from base + offset (base the same for the whole wave, offset in bytes per lane)
@@ -110,7 +111,7 @@ __device__ __forceinline__ void tile_store(const TileArgs& a, const f32x16 (&acc
                         const int j = n0 + wn * HALF + tn * 32 + r32;
                         const float gate = round_through<__bf16>(acc[tm][tn][v]);
                         const float up = round_through<__bf16>(acc[tm][tn + TN / 2][v]);
-                        if (m < a.M && j < inner)
+                        if (m < a.M && j < min(inner, n0 + a.cols_per_wg))
                             ((__bf16*)a.y)[(int64_t)m * a.y_stride + j] = (__bf16)(gate / (1.f + __expf(-gate)) * up);
                     }
         }
@@ -127,7 +128,7 @@ __device__ __forceinline__ void tile_store(const TileArgs& a, const f32x16 (&acc
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int m = m_wave + tm * 32 + 8 * (v / 4) + 4 * half + v % 4;
-                if (m >= a.M || n >= a.N) continue;
+                if (m >= a.M || n >= min(a.N, n0 + a.cols_per_wg)) continue;
                 const float val = acc[tm][tn][v] + b;
                 if (a.mode == TL_PARTIAL) a.partial[((int64_t)blockIdx.y * a.M + m) * a.N + n] = val;
                 else if (a.mode == TL_PLAIN_F32) ((float*)a.y)[(int64_t)m * a.y_stride + n] = val;
@@ -139,12 +140,15 @@ __device__ __forceinline__ void tile_store(const TileArgs& a, const f32x16 (&acc
 // The row of W that lies in LDS row r of the workgroup's W tile: BN rows in a row from n0, or
 // (gated) for every wave's part half as many gate rows followed by the up rows that belong to them,
 // so that a lane holds both of an output.  Kept inside the weight.
+// A workgroup that takes fewer columns than its tile has fetches the row of its last column again
+// in place of the others (the same line, found in the cache).
 template <int PART>
 __device__ __forceinline__ int tile_w_row(const TileArgs& a, int n0, int r) {
-    if (a.mode != TL_GATED) return min(n0 + r, a.N - 1);
+    if (a.mode != TL_GATED) return min(n0 + min(r, a.cols_per_wg - 1), a.N - 1);
     constexpr int HALF = PART / 2;
     const int inner = a.N / 2, part = r / PART, q = r % PART;
-    return q < HALF ? min(n0 + part * HALF + q, inner - 1) : min(n0 + part * HALF + q - HALF, inner - 1) + inner;
+    const int col = min(part * HALF + (q < HALF ? q : q - HALF), a.cols_per_wg - 1);
+    return min(n0 + col, inner - 1) + (q < HALF ? 0 : inner);
 }
 
 // Four waves that fetch and multiply: every wave brings its share of both tiles, STAGES chunks in
@@ -163,7 +167,7 @@ linear_tile_kernel(const TileArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / NVA_WAVE), lane = threadIdx.x % NVA_WAVE;
     const int wm = wave / WN, wn = wave % WN;
     const int m0 = blockIdx.z * BM;
-    const int n0 = a.mode == TL_GATED ? blockIdx.x * (BN / 2) : blockIdx.x * BN;
+    const int n0 = blockIdx.x * a.cols_per_wg;
     const int chunks_total = a.K / TL_BK;
     const int chunk_begin = blockIdx.y * a.chunks_per_range;
     const int chunks = min(a.chunks_per_range, chunks_total - chunk_begin);
@@ -234,7 +238,7 @@ linear_tile_fed_kernel(const TileArgs a) {
     extern __shared__ __attribute__((aligned(1024))) char tl_lds[];     // [SX] x tiles, then [SW] W tiles
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / NVA_WAVE), lane = threadIdx.x % NVA_WAVE;
     const int m0 = blockIdx.z * BM;
-    const int n0 = a.mode == TL_GATED ? blockIdx.x * (BN / 2) : blockIdx.x * BN;
+    const int n0 = blockIdx.x * a.cols_per_wg;
     const int chunks_total = a.K / TL_BK;
     const int chunk_begin = blockIdx.y * a.chunks_per_range;
     const int chunks = min(a.chunks_per_range, chunks_total - chunk_begin);
@@ -327,7 +331,10 @@ NVA_EXPORT int nva_linear_tile_shapes() { return (int)(sizeof(tile_shapes) / siz
 
 NVA_EXPORT int nva_linear_tile_bf16(const void* x, int64_t x_stride, const void* w, int64_t w_stride, const void* bias,
                                     void* y, int64_t y_stride, float* partial, int mode, int64_t M, int64_t N, int64_t K,
-                                    int shape, int stages, int ranges, int* ranges_used, hipStream_t stream) {
+                                    int shape, int stages, int ranges, int cols_per_wg, int* ranges_used, hipStream_t stream) {
+    // cols_per_wg: 0, or the columns of y one workgroup takes where that is to be fewer than its tile
+    // has (64 of the gated form's 128 rows of W, else 128 or 256): more, lighter workgroups, so that
+    // a weight's rows can be shared out evenly over the CUs.
     if (M == 0 || N == 0) return 0;
     if (M < 0 || N < 0 || K <= 0 || K % TL_BK || M > 0x7fffffff || N > 0x7fffffff ||
         (M * x_stride + K) * 2 > 0xffffffffLL || (N * w_stride + K) * 2 > 0xffffffffLL) {
@@ -361,7 +368,11 @@ NVA_EXPORT int nva_linear_tile_bf16(const void* x, int64_t x_stride, const void*
     a.chunks_per_range = (chunks + ranges - 1) / ranges;
     const int real_ranges = (chunks + a.chunks_per_range - 1) / a.chunks_per_range;
     const int64_t cols = mode == TL_GATED ? N / 2 : N;
-    const int per_wg = mode == TL_GATED ? sh.bn / 2 : sh.bn;
+    const int tile_cols = mode == TL_GATED ? sh.bn / 2 : sh.bn;
+    if (cols_per_wg < 0 || cols_per_wg > tile_cols) return nva_fail("linear_tile: %d columns per workgroup of a tile of %d", cols_per_wg, tile_cols);
+    const int per_wg = cols_per_wg ? cols_per_wg : tile_cols;
+    a.cols_per_wg = per_wg;
+    if ((cols + per_wg - 1) / per_wg > 0x7fffffff) return nva_fail("linear_tile: too many workgroups");
     const dim3 grid((unsigned)((cols + per_wg - 1) / per_wg), (unsigned)real_ranges, (unsigned)((M + sh.bm - 1) / sh.bm));
 #define LAUNCH_KERNEL(KERNEL, THREADS)                                                                                 \
     do {                                                                                                               \

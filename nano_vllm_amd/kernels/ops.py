@@ -220,6 +220,7 @@ class HipKernels:
         # Rows up to which the bfloat16 product runs on the engine's own kernels.
         props = torch.cuda.get_device_properties(self.device)
         cus = props.multi_processor_count
+        self.cus = cus
         self.own_matmul_rows = 16           # bfloat16 products with more rows go to the library ...
         self.skinny_max_rows = 64           # ... unless the weight is small (see _own_rows); the kernel's limit
         self.small_weight_bytes = 64 << 20
@@ -244,7 +245,8 @@ class HipKernels:
         self.product_choice = recorded_product_choices(props.name)
         self.choice_margin = 0.10           # the rule's kernel stays unless the other is faster by more than this
         self.tile_for_wide_weights = True   # False: the rule never names the LDS-tiled kernel (tests)
-        self.tile_shape = None              # (shape, stages, ranges) forced on the LDS-tiled kernel (tests)
+        self.tile_shape = None              # (shape, stages, ranges[, columns per workgroup]) forced on the LDS-tiled kernel (tests)
+        self.tile_even_shares = True        # False: the LDS-tiled kernel's workgroups always take whole tiles (tests)
         self.fuse_split_sums = True         # False: every product is finished by its own pass
         # False: attention always runs the general kernel (tests compare the two)
         self.mfma_attention = True
@@ -651,18 +653,39 @@ class HipKernels:
         LDS holds, and, where the result may stay as partial sums, k cut into as many ranges as give
         about one workgroup per CU."""
         if self.tile_shape is not None:
-            return self.tile_shape
+            return tuple(self.tile_shape) + (0,) * (4 - len(self.tile_shape))
         shape, stages = (1, 3) if m <= 64 else (2, 3) if m <= 128 else (3, 4)     # (64 rows: two workgroups fit a CU)
         tiles = ((n // 2 if gated else n) + (63 if gated else 127)) // (64 if gated else 128)
         ranges = 1
         if may_split and not gated:
             ranges = max(1, min(self.teams // max(tiles, 1), k // 256))
-        return shape, stages, ranges
+        return shape, stages, ranges, self._tile_cols(m, n // 2 if gated else n, 64 if gated else 128, ranges)
+
+    def _tile_cols(self, m: int, cols: int, tile_cols: int, ranges: int) -> int:
+        """Columns of the result that a workgroup of the LDS-tiled kernel takes (0: its whole tile).  A CU
+        draws its share of the memory's bandwidth and no more, so a weight is streamed fastest when every
+        CU gets as many of its rows as every other: where whole tiles would make a second round that
+        few CUs work in, or leave many CUs idle, the workgroups take as many columns each as shares
+        the weight out evenly over the CUs in as many rounds (14B gate/up, 272 tiles on 256 CUs: 84
+        instead of 105 µs at 64 rows, 153 instead of 164 at 256; 32B, 400 tiles: 111 instead of 116; 4B,
+        152 tiles: 25 instead of 29).  Not where three quarters of the CUs have a tile anyway (8B
+        gate/up, 192 tiles: the same time either way), not for a single round of more than 128 rows of x
+        (every workgroup fetches all of x, and more workgroups fetch it more often: 72 instead of 65 µs
+        there at 256 rows), and not for many rounds, which the hardware hands out evenly by itself (the
+        head, 1187 tiles: 3 % slower)."""
+        if self.tile_even_shares is False or ranges > 1:
+            return 0
+        tiles = (cols + tile_cols - 1) // tile_cols
+        rounds = (tiles + self.cus - 1) // self.cus
+        if tiles % self.cus == 0 or rounds > 2 or (rounds == 1 and (m > 128 or 10 * tiles > 7 * self.cus)):
+            return 0
+        share = ((cols + rounds * self.cus - 1) // (rounds * self.cus) + 7) // 8 * 8
+        return share if share < tile_cols else 0
 
     def _linear_tile(self, x, xs, weight, ws, bias, out, os_, out_float32, swiglu, m, n, k, defer=False):
         """The LDS-tiled kernel for 17 rows and more (see _linear_skinny for the arguments)."""
         gated = bool(swiglu and bias is None and not defer)
-        shape, stages, ranges = self._tile_plan(m, n, k, gated, may_split=not gated and not out_float32)
+        shape, stages, ranges, cols = self._tile_plan(m, n, k, gated, may_split=not gated and not out_float32)
         if swiglu and not gated:
             raise KernelError("linear_tile: the gated form takes no bias and is never deferred")
         if ranges == 1:
@@ -673,13 +696,13 @@ class HipKernels:
             mode = 2 if gated else 1 if out_float32 else 0
             library.call("gemm_tile", "bf16", "nva_linear_tile", _p(x), c_i64(xs), _p(weight), c_i64(ws), _p(bias), _p(out),
                          c_i64(os_), None, c_i32(mode), c_i64(m), c_i64(n), c_i64(k), c_i32(shape), c_i32(stages), c_i32(1),
-                         None, self._stream())
+                         c_i32(cols), None, self._stream())
             return out
         scratch = torch.empty(ranges * m * n, dtype=torch.float32, device=x.device)
         used = ctypes.c_int(0)
         library.call("gemm_tile", "bf16", "nva_linear_tile", _p(x), c_i64(xs), _p(weight), c_i64(ws), None, None, c_i64(0),
                      _p(scratch), c_i32(3), c_i64(m), c_i64(n), c_i64(k), c_i32(shape), c_i32(stages), c_i32(ranges),
-                     ctypes.byref(used), self._stream())
+                     c_i32(cols), ctypes.byref(used), self._stream())
         sums = SplitSum(self, scratch, used.value, m, n, bias)
         if defer:
             return sums

@@ -97,3 +97,24 @@ def test_the_record_of_measured_choices_survives_a_round_trip(tmp_path, monkeypa
     record.write_text("not json")
     monkeypatch.setattr(ops, "_product_choices", {})
     assert ops.recorded_product_choices("a GPU") == {}           # an unreadable record: measured again
+
+
+def test_the_tiled_kernels_workgroups_share_a_weight_out_evenly():
+    """Where whole tiles of the LDS-tiled kernel would leave many CUs idle or make a second round that
+    few CUs work in, a workgroup takes as many columns as shares the weight out evenly; where most CUs
+    have a tile, where a single round has more than 128 rows of x, and where there are many rounds,
+    whole tiles stay."""
+    from nano_vllm_amd.kernels.ops import HipKernels
+    k = HipKernels.__new__(HipKernels)
+    k.cus, k.tile_even_shares = 256, True
+    assert k._tile_cols(64, 17408, 64, 1) == 40          # 14B gate/up: 272 tiles, two rounds -> 436 workgroups of 40
+    assert k._tile_cols(256, 17408, 64, 1) == 40
+    assert k._tile_cols(64, 25600, 64, 1) == 56          # 32B gate/up: 400 tiles
+    assert k._tile_cols(64, 9728, 64, 1) == 40           # 4B gate/up: 152 tiles, one round
+    assert k._tile_cols(256, 9728, 64, 1) == 0           # ... but not with 256 rows of x
+    assert k._tile_cols(64, 12288, 64, 1) == 0           # 8B gate/up: 192 of 256 CUs have a tile
+    assert k._tile_cols(64, 151936, 128, 1) == 0         # the head: five rounds
+    assert k._tile_cols(64, 16384, 64, 1) == 0           # 256 tiles: even as they are
+    assert k._tile_cols(64, 17408, 64, 4) == 0           # k cut into ranges: the workgroups are counted otherwise
+    k.tile_even_shares = False
+    assert k._tile_cols(64, 17408, 64, 1) == 0

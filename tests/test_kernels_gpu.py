@@ -881,12 +881,15 @@ def test_the_lds_tiled_product_at_drawn_shapes(hip, seed):
     n = 2 * rng.choice([rng.randint(1, 150), rng.randint(500, 4500)])
     k = 64 * rng.choice([rng.randint(1, 8), rng.randint(20, 90)])
     ranges = rng.choice([1, 1, rng.randint(2, 9)])
+    # columns of the result per workgroup: the whole tile, or fewer (a multiple of 8 as the engine
+    # draws them, or any number); the gated form's tile has half as many columns as rows of W
+    cols = rng.choice([0, 0, 8 * rng.randint(1, bn // 16), rng.randint(1, bn // 2)])
     kern = hip[torch.bfloat16]
     x, w = _rand((m, k), torch.bfloat16, 5100 + seed), _rand((n, k), torch.bfloat16, 5200 + seed, 0.05)
     b = _rand((n,), torch.bfloat16, 5300 + seed)
     want = x.double() @ w.double().T
-    what = f"m {m} n {n} k {k} shape {shape} stages {stages} ranges {ranges}"
-    kern.tile_shape = (shape, stages, ranges)
+    what = f"m {m} n {n} k {k} shape {shape} stages {stages} ranges {ranges} columns {cols}"
+    kern.tile_shape = (shape, stages, ranges, cols)
     try:
         out = torch.empty((m, n), dtype=torch.bfloat16, device=DEV)
         kern._linear_tile(x, k, w, k, b, out, n, False, False, m, n, k)
@@ -900,7 +903,7 @@ def test_the_lds_tiled_product_at_drawn_shapes(hip, seed):
             sums = got.sums[:got.splits * m * n].view(got.splits, m, n).double().sum(0)
             assert bool(((sums - want).abs() <= bound).all()), what + " partial sums"
         if shape != 0:
-            kern.tile_shape = (shape, stages, 1)
+            kern.tile_shape = (shape, stages, 1, cols)
             gated = torch.empty((m, n // 2), dtype=torch.bfloat16, device=DEV)
             kern._linear_tile(x, k, w, k, None, gated, n // 2, False, True, m, n, k)
             y = want.float().to(torch.bfloat16).float()
