@@ -146,6 +146,46 @@ def test_layer_sizes_of_the_named_shapes(real_size_folder, name, dtype):
     r.kernels.check_faults()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_that_lie_beyond_four_gibibytes_of_a_layers_keys(real_size_folder, dtype):
+    """A cache as large as a serving engine's: pages of 256 tokens of the 8B shape's 8 kv heads of
+    128 are 512 KiB of a layer's keys each (1 MiB in float32), so page 8192 begins 2^31 elements and
+    4 GiB (8 GiB) into the tensor.  With the first 8200 pages held by another request, a request's pages lie beyond
+    that: its keys and values are written there, by a prompt's portions and by single tokens, and
+    read from there, and the logits are those of the plain implementation."""
+    folder = real_size_folder("qwen3-8b")
+    first = 8200
+    r = ModelRunner.from_folder(folder, dtype=dtype, page_size=256, num_pages=first + 6, max_requests=4, quiet=True,
+                                enable_prefix_caching=False)
+    pool = r.cache.pools[0]
+    r.cache.admit("holds the first pages")
+    r.cache.reserve("holds the first pages", first * 256)
+    assert sorted(r.cache.table("holds the first pages", 0)) == list(range(first))
+    toks = H.random_tokens(2048, 300, 7)
+    pcfg, w = plain.read_folder(folder)
+    want = plain.logits(w, pcfg, toks, None if dtype == "float32" else "bfloat16")
+    tol = 2e-5 if dtype == "float32" else 2e-2
+    for portions in ([300 - 32] + [1] * 32, [250, 2, 7, 41]):
+        r.cache.admit("x")
+        out, pos = [], 0
+        for n in portions:
+            r.cache.reserve("x", pos + n)
+            assert min(r.cache.table("x", 0)) >= first
+            out.append(r.step([StepEntry("x", toks[pos:pos + n], pos, list(range(n)))]).float().cpu())
+            pos += n
+        r.cache.release("x")
+        assert H.rel_err(torch.cat(out), want) < tol, portions
+    # two requests in one step: single tokens of one beside a portion of the other
+    reqs = {"a": H.random_tokens(2048, 290, 21), "b": H.random_tokens(2048, 270, 22)}
+    got = H.run_mixed(r, reqs, seed=4)
+    for rid, t in reqs.items():
+        assert H.rel_err(got[rid], plain.logits(w, pcfg, t, None if dtype == "float32" else "bfloat16")) < tol, rid
+    r.kernels.check_faults()
+    r.cache.release("holds the first pages")
+    r.cache.check()
+    assert pool.num_free == first + 6
+
+
 def test_two_engines_on_one_model_choose_the_same_product_kernels(real_size_folder, tmp_path, monkeypatch):
     """The product kernels for 17 to 256 rows are measured once and recorded: a second engine, and
     a second process (its table emptied here, so that it comes from the record), run the same
