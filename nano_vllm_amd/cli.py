@@ -26,7 +26,7 @@ def add_engine_options(ap: argparse.ArgumentParser) -> None:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--schedule", default="prefill_first", choices=["prefill_first", "mixed"])
     ap.add_argument("--no-prefix-caching", action="store_true")
-    ap.add_argument("--decode-burst", type=int, default=8, help="decode steps in a row without the host (1: never)")
+    ap.add_argument("--decode-burst", type=int, default=16, help="decode steps in a row without the host (1: never)")
     ap.add_argument("--random-weights", type=int, default=None, metavar="SEED",
                     help="draw the weights on the device from this seed: the folder needs config.json only")
 

@@ -28,7 +28,7 @@ class EngineConfig:
     schedule: str = "prefill_first"         # the reference's policy, or "mixed"
     enable_prefix_caching: bool = True
     device: str = "cuda:0"
-    decode_burst: int = 8                   # decode steps in a row without the host, while no request waits (1: never)
+    decode_burst: int = 16                  # decode steps in a row without the host, while no request waits (1: never)
     random_weights: Optional[int] = None    # a seed: the folder needs config.json only, weights are drawn on the device
     measure_products: bool = True           # False: product kernels for 17-256 rows by rule and record only, nothing is timed at start-up
 

@@ -172,7 +172,7 @@ class LLMEngine:
                 if last:
                     sampled.append(seq)
             burst = self._burst_steps(seqs, entries, is_prefill)
-            decoded = len(seqs)                  # tokens a decode step reports: one per request and step of a burst
+            decoded = len(seqs)                  # tokens a decode step reports: one per request and step of a burst that it is still in
             if burst > 1:
                 rows = self.runner.decode_burst(
                     entries, burst, self.sampler, [s.temperature for s in seqs],
@@ -183,7 +183,8 @@ class LLMEngine:
                         s.num_scheduled_tokens = 1
                     self.scheduler.postprocess([s for s, _ in live], [t for _, t in live])
                     self.stats["decode_tokens"] += len(live)
-                decoded = len(seqs) * burst
+                    decoded += len(live)
+                decoded -= len(seqs)
                 self.stats["decode_tokens"] -= len(seqs)            # the first row is counted below
             else:
                 logits = self.runner.step(entries)
@@ -212,7 +213,7 @@ class LLMEngine:
     def _burst_steps(self, seqs, entries, is_prefill) -> int:
         """How many decode steps to run in a row without the host: more than one only while
         no request waits, every request of the step decodes, the captured steps take the batch,
-        and pages for all the steps can be reserved; never past a request's last token."""
+        and pages for all the steps can be reserved."""
         want = self.config.decode_burst
         if want <= 1 or is_prefill or self.scheduler.waiting or not seqs:
             return 1
@@ -224,16 +225,23 @@ class LLMEngine:
         for s in seqs:
             if s.num_cached_tokens + 1 != s.num_tokens:
                 return 1
-            want = min(want, s.max_tokens - s.num_completion_tokens, self.config.max_model_len - s.num_tokens)
-        if want <= 1:
-            return 1
-        # all requests or none: a request must not keep pages for steps that will not run
-        wanted = [(s.seq_id, s.num_tokens + want - 1, s.num_tokens - 1) for s in seqs]
-        if not runner.cache.can_reserve_all(wanted):
-            return 1
-        for request, new_len, first_query in wanted:
-            runner.cache.reserve(request, new_len, first_query=first_query)
-        return want
+        left = [s.max_tokens - s.num_completion_tokens for s in seqs]
+        room = min(self.config.max_model_len - s.num_tokens for s in seqs)
+        # A burst may run past the last token of some of its requests, as it runs past an eos token:
+        # their rows are computed and dropped, and the host is asked once per burst and not once per
+        # request that ends.  It never runs past the last token of all of them, nor past the longest
+        # sequence the model takes; where the pool has no pages for that, it ends with the first
+        # request that ends.
+        for steps in dict.fromkeys((min(want, max(left), room), min(want, min(left), room))):
+            if steps <= 1:
+                break
+            # all requests or none: a request must not keep pages for steps that will not run
+            wanted = [(s.seq_id, s.num_tokens + steps - 1, s.num_tokens - 1) for s in seqs]
+            if runner.cache.can_reserve_all(wanted):
+                for request, new_len, first_query in wanted:
+                    runner.cache.reserve(request, new_len, first_query=first_query)
+                return steps
+        return 1
 
     def generate(self, prompts: Seq[Union[str, List[int]]],
                  sampling_params: Union[SamplingParams, Seq[SamplingParams], None] = None,
